@@ -152,6 +152,17 @@ __device__ __forceinline__ float apply_act(float x, int act) {
     }
 }
 
+// act(g) * u, or the clamped gate (kinds and fields: PtaGate in pta_kernels.h), in 32-bit
+template <typename Gate>
+__device__ __forceinline__ float gate_value(float g, float u, int act, const Gate& how) {
+    if (how.kind == 1) {
+        g = fminf(g, how.limit);
+        u = fminf(fmaxf(u, -how.limit), how.limit);
+        return g / (1.0f + expf(-how.alpha * g)) * (u + 1.0f);
+    }
+    return apply_act(g, act) * u;
+}
+
 // ---- host side ---------------------------------------------------------
 // Entry points return 0 on success; otherwise pta_last_error() holds the reason.
 int pta_fail(const char* fmt, ...);

@@ -30,6 +30,38 @@ extern "C" int pta_embed(void* out, const void* table, const int* ids, int M, in
     return pta_check_launch("embed");
 }
 
+// A scaled token embedding plus a learned vector for the token's position, formed and left in 32-bit (the start of a
+// stream that is held so).  Positions past the table's end read its last row: the caller refuses them beforehand.
+template <typename T>
+__global__ void embed_pos_kernel(float* __restrict__ out, const T* __restrict__ table, const int* __restrict__ ids,
+                                 const T* __restrict__ pos_table, const int* __restrict__ token_pos, float scale, int H,
+                                 int positions) {
+    const int m = blockIdx.x;
+    const T* src = table + (long)ids[m] * H;
+    const T* pr = pos_table ? pos_table + (long)min(max(token_pos[m], 0), positions - 1) * H : nullptr;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        float v = Io<T>::ld(src + i) * scale;
+        if (pr) v += Io<T>::ld(pr + i);
+        out[(long)m * H + i] = v;
+    }
+}
+
+extern "C" int pta_embed_pos(float* out, const void* table, const int* ids, const void* pos_table, const int* token_pos,
+                             float scale, int M, int H, int positions, int dtype, void* stream) {
+    PTA_REQUIRE(M > 0 && H > 0 && out && table && ids, "embed_pos: M=%d H=%d must be positive and pointers given", M, H);
+    PTA_REQUIRE(!pos_table || (token_pos && positions > 0), "embed_pos: a position table needs positions");
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == PTA_F32)
+        hipLaunchKernelGGL(embed_pos_kernel<float>, dim3(M), dim3(256), 0, s, out, (const float*)table, ids,
+                           (const float*)pos_table, token_pos, scale, H, positions);
+    else if (dtype == PTA_BF16)
+        hipLaunchKernelGGL(embed_pos_kernel<bf16_t>, dim3(M), dim3(256), 0, s, out, (const bf16_t*)table, ids,
+                           (const bf16_t*)pos_table, token_pos, scale, H, positions);
+    else
+        return pta_fail("embed_pos: unknown dtype %d", dtype);
+    return pta_check_launch("embed_pos");
+}
+
 // y = (x - mean) / sqrt(var + eps) * w + b, biased variance (torch.nn.LayerNorm as built at
 // src/transformers/models/falcon/modeling_falcon.py:603-612, :843).  w and b are 32-bit.
 template <typename T>

@@ -91,3 +91,42 @@ extern "C" int pta_glu(void* out, const void* gate, const void* up, long in_ld, 
         hipLaunchKernelGGL(glu_kernel<bf16_t>, grid, dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)gate, (const bf16_t*)up, in_ld, F, n, kind, alpha, limit);
     return pta_check_launch("glu");
 }
+
+// PolyNorm (see pta_kernels.h): one workgroup per row, the three mean squares in one pass, the row read again for the
+// output.  Sums are 32-bit, in an order that depends on the row's length alone.
+template <typename T>
+__global__ __launch_bounds__(256) void polynorm_kernel(T* __restrict__ out, const T* __restrict__ z, long z_ld,
+                                                       const float* __restrict__ coef, float eps, int F) {
+    __shared__ float red[16];
+    const T* zr = z + (long)blockIdx.x * z_ld;
+    float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    for (int i = threadIdx.x; i < F; i += blockDim.x) {
+        const float v = Io<T>::ld(zr + i), v2 = v * v;
+        s1 += v2;
+        s2 += v2 * v2;
+        s3 += v2 * v2 * v2;
+    }
+    const float inv_f = 1.0f / (float)F;
+    const float r1 = coef[0] / sqrtf(block_sum(s1, red) * inv_f + eps);
+    const float r2 = coef[1] / sqrtf(block_sum(s2, red) * inv_f + eps);
+    const float r3 = coef[2] / sqrtf(block_sum(s3, red) * inv_f + eps);
+    const float e = coef[3];
+    T* orow = out + (long)blockIdx.x * F;
+    for (int i = threadIdx.x; i < F; i += blockDim.x) {
+        const float v = Io<T>::ld(zr + i), v2 = v * v;
+        Io<T>::st(orow + i, r1 * v + r2 * v2 + r3 * (v2 * v) + e);
+    }
+}
+
+extern "C" int pta_polynorm(void* out, const void* z, long z_ld, const float* coef, float eps, int M, int F, int dtype,
+                            void* stream) {
+    PTA_REQUIRE(M > 0 && F > 0 && out && z && coef && z_ld >= F, "polynorm: sizes must be positive and pointers given");
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == PTA_F32)
+        hipLaunchKernelGGL(polynorm_kernel<float>, dim3(M), dim3(256), 0, s, (float*)out, (const float*)z, z_ld, coef, eps, F);
+    else if (dtype == PTA_BF16)
+        hipLaunchKernelGGL(polynorm_kernel<bf16_t>, dim3(M), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)z, z_ld, coef, eps, F);
+    else
+        return pta_fail("polynorm: unknown dtype %d", dtype);
+    return pta_check_launch("polynorm");
+}

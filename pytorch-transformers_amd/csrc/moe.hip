@@ -3,6 +3,7 @@
 //   z = W_r h (32-bit); s = score(z) (sigmoid, or softmax over the experts); the `top` largest s are taken;
 //   weights = s / (sum of the taken s + 1e-20) * scale   (or the taken s times scale, unnormalised);
 //   out = sum over the taken experts e of weight_e * D_e (act(G_e h) * (U_e h))
+//   (z may have a bias added; in place of act(g) * u an expert may have the clamped gate of PtaGate, pta_kernels.h)
 //
 // Expert matrices are held stacked: gate_up [E, 2F, H] (an expert's gate rows, then its up rows) and down [E, H, F].
 //
@@ -78,7 +79,8 @@ __device__ __forceinline__ void wave_dots(const T* __restrict__ w, long row_ld, 
 template <typename T>
 __global__ __launch_bounds__(1024) void moe_route_kernel(int* __restrict__ ids, float* __restrict__ wts,
                                                         const T* __restrict__ h, long h_ld, const float* __restrict__ Wr,
-                                                        int H, int E, int top, int score_kind, int normalise, float scale) {
+                                                        const float* __restrict__ br, int H, int E, int top, int score_kind,
+                                                        int normalise, float scale) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
     float* x_s = sm;       // [H]
     float* s_s = sm + H;   // [E]
@@ -87,7 +89,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(int* __restrict__ ids, 
     __syncthreads();
     for (int e = wave; e < E; e += nw) {
         const float z = wave_dot<float>(Wr + (long)e * H, x_s, H, lane);
-        if (lane == 0) s_s[e] = z;
+        if (lane == 0) s_s[e] = br ? z + br[e] : z;
     }
     __syncthreads();
     if (wave != 0) return;
@@ -129,7 +131,7 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(int* __restrict__ ids, 
     }
 }
 
-extern "C" int pta_moe_route(int* ids, float* wts, const void* h, long h_ld, const float* Wr, int M, int H, int E, int top,
+extern "C" int pta_moe_route(int* ids, float* wts, const void* h, long h_ld, const float* Wr, const float* br, int M, int H, int E, int top,
                              int score_kind, int normalise, float scale, int dtype, void* stream) {
     PTA_REQUIRE(M > 0 && H > 0 && E > 0 && top > 0, "moe_route: sizes must be positive");
     PTA_REQUIRE(top <= E && top <= 64 && E <= 2048, "moe_route: %d experts per token of %d (at most 64 of at most 2048)", top, E);
@@ -141,9 +143,9 @@ extern "C" int pta_moe_route(int* ids, float* wts, const void* h, long h_ld, con
     const size_t lds = (size_t)(H + E) * sizeof(float);
     const dim3 block(E >= 16 ? 1024 : E >= 8 ? 512 : 256);  // a wave an expert where there are that many
     if (dtype == PTA_F32)
-        hipLaunchKernelGGL(moe_route_kernel<float>, dim3(M), block, lds, s, ids, wts, (const float*)h, h_ld, Wr, H, E, top, score_kind, normalise, scale);
+        hipLaunchKernelGGL(moe_route_kernel<float>, dim3(M), block, lds, s, ids, wts, (const float*)h, h_ld, Wr, br, H, E, top, score_kind, normalise, scale);
     else
-        hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(M), block, lds, s, ids, wts, (const bf16_t*)h, h_ld, Wr, H, E, top, score_kind, normalise, scale);
+        hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(M), block, lds, s, ids, wts, (const bf16_t*)h, h_ld, Wr, br, H, E, top, score_kind, normalise, scale);
     return pta_check_launch("moe_route");
 }
 
@@ -152,7 +154,7 @@ extern "C" int pta_moe_route(int* ids, float* wts, const void* h, long h_ld, con
 template <typename T>
 __global__ __launch_bounds__(256) void moe_up_kernel(T* __restrict__ act_out, const T* __restrict__ h, long h_ld,
                                                      const T* __restrict__ gate_up, const int* __restrict__ ids, int H,
-                                                     int F, int top, int act) {
+                                                     int F, int top, int act, PtaGate gate) {
     extern __shared__ __attribute__((aligned(16))) float x_s[];  // [H]
     const int pair = blockIdx.x, m = pair / top, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int e = ids[pair];
@@ -172,7 +174,7 @@ __global__ __launch_bounds__(256) void moe_up_kernel(T* __restrict__ act_out, co
 #pragma unroll
         for (int r = 1; r < 4; ++r)
             if (lane == r) { gv = g[r]; uv = u[r]; }
-        Io<T>::st(act_out + (long)pair * F + f0 + lane, apply_act(Io<T>::round(gv), act) * Io<T>::round(uv));
+        Io<T>::st(act_out + (long)pair * F + f0 + lane, gate_value(Io<T>::round(gv), Io<T>::round(uv), act, gate));
     }
 }
 
@@ -205,7 +207,9 @@ __global__ __launch_bounds__(256) void moe_down_kernel(T* __restrict__ out, cons
 
 // act_out [M * top, F]; h [M, H] rows h_ld apart; gate_up [E, 2F, H]; ids [M, top]
 extern "C" int pta_moe_up(void* act_out, const void* h, long h_ld, const void* gate_up, const int* ids, int M, int H, int F,
-                          int top, int act, int dtype, void* stream) {
+                          int top, int act, const PtaGate* gate_how, int dtype, void* stream) {
+    const PtaGate gate = gate_how ? *gate_how : PtaGate{PTA_GLU_SILU, 1.f, 0.f};
+    PTA_REQUIRE(gate.kind == PTA_GLU_SILU || gate.kind == PTA_GLU_CLAMPED, "moe_up: a gate of kind %d is not built", gate.kind);
     PTA_REQUIRE(M > 0 && H > 0 && F > 0 && top > 0 && act_out && h && gate_up && ids && h_ld >= H, "moe_up: sizes must be positive and pointers given");
     PTA_REQUIRE(pta_act_known(act), "moe_up: unknown activation %d", act);
     PTA_REQUIRE((size_t)H * 4 <= 64 * 1024 && (F + MOE_ROWS - 1) / MOE_ROWS <= 65535, "moe_up: sizes beyond one launch");
@@ -213,9 +217,9 @@ extern "C" int pta_moe_up(void* act_out, const void* h, long h_ld, const void* g
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid((unsigned)((long)M * top), (F + MOE_ROWS - 1) / MOE_ROWS);
     if (dtype == PTA_F32)
-        hipLaunchKernelGGL(moe_up_kernel<float>, grid, dim3(256), (size_t)H * 4, s, (float*)act_out, (const float*)h, h_ld, (const float*)gate_up, ids, H, F, top, act);
+        hipLaunchKernelGGL(moe_up_kernel<float>, grid, dim3(256), (size_t)H * 4, s, (float*)act_out, (const float*)h, h_ld, (const float*)gate_up, ids, H, F, top, act, gate);
     else
-        hipLaunchKernelGGL(moe_up_kernel<bf16_t>, grid, dim3(256), (size_t)H * 4, s, (bf16_t*)act_out, (const bf16_t*)h, h_ld, (const bf16_t*)gate_up, ids, H, F, top, act);
+        hipLaunchKernelGGL(moe_up_kernel<bf16_t>, grid, dim3(256), (size_t)H * 4, s, (bf16_t*)act_out, (const bf16_t*)h, h_ld, (const bf16_t*)gate_up, ids, H, F, top, act, gate);
     return pta_check_launch("moe_up");
 }
 
@@ -384,7 +388,7 @@ __global__ __launch_bounds__(256) void moe_grouped_up_kernel(bf16_t* __restrict_
                                                              long x_ld, const bf16_t* __restrict__ gate_up,
                                                              const int* __restrict__ sorted_pair,
                                                              const int* __restrict__ tile_expert, int H, int F, int top,
-                                                             int act, int tiles) {
+                                                             int act, PtaGate gate, int tiles) {
     __shared__ __attribute__((aligned(16))) bf16_t lds[2 * MOE_TILE * MOE_XROW];
     int tile, fb;
     if (!moe_item(tiles, (F + 127) / 128, &tile, &fb)) return;
@@ -411,7 +415,7 @@ __global__ __launch_bounds__(256) void moe_grouped_up_kernel(bf16_t* __restrict_
             float y[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                y[j] = apply_act(round_to_bf16(acc[half][tt][j]), act) * round_to_bf16(acc[2 + half][tt][j]);
+                y[j] = gate_value(round_to_bf16(acc[half][tt][j]), round_to_bf16(acc[2 + half][tt][j]), act, gate);
             const int f = f0 + half * 16 + 4 * gq;
             moe_store4(act_sorted + slot * F + f, f, F, y[0], y[1], y[2], y[3]);
         }
@@ -466,7 +470,10 @@ extern "C" int pta_moe_grouped_slots(int pairs, int E) { return (pairs + E * (MO
 // act_sorted [slots, F], y_sorted [slots, H] are the caller's scratch (slots = pta_moe_grouped_slots(M * top, E)).
 extern "C" int pta_moe_grouped(void* out, const void* x, long x_ld, const void* gate_up, const void* down, const int* ids,
                                const float* wts, int* sorted_pair, int* slot_of_pair, int* tile_expert, void* act_sorted,
-                               void* y_sorted, int M, int H, int F, int E, int top, int act, void* stream) {
+                               void* y_sorted, int M, int H, int F, int E, int top, int act, const PtaGate* gate_how,
+                               void* stream) {
+    const PtaGate gate = gate_how ? *gate_how : PtaGate{PTA_GLU_SILU, 1.f, 0.f};
+    PTA_REQUIRE(gate.kind == PTA_GLU_SILU || gate.kind == PTA_GLU_CLAMPED, "moe_grouped: a gate of kind %d is not built", gate.kind);
     PTA_REQUIRE(M > 0 && H > 0 && F > 0 && E > 0 && top > 0, "moe_grouped: sizes must be positive");
     PTA_REQUIRE(H % 64 == 0 && F % 64 == 0 && x_ld % 8 == 0, "moe_grouped: features (%d) and expert size (%d) must be multiples of 64", H, F);
     PTA_REQUIRE(out && x && gate_up && down && ids && wts && sorted_pair && slot_of_pair && tile_expert && act_sorted && y_sorted,
@@ -483,7 +490,7 @@ extern "C" int pta_moe_grouped(void* out, const void* x, long x_ld, const void* 
                        ids, (int)pairs, E, slots, tiles);
     auto grid_for = [&](int blocks) { return dim3((unsigned)(((long)tiles * blocks + 7) / 8 * 8)); };
     hipLaunchKernelGGL(moe_grouped_up_kernel, grid_for((F + 127) / 128), dim3(256), 0, s, (bf16_t*)act_sorted, (const bf16_t*)x,
-                       x_ld, (const bf16_t*)gate_up, sorted_pair, tile_expert, H, F, top, act, tiles);
+                       x_ld, (const bf16_t*)gate_up, sorted_pair, tile_expert, H, F, top, act, gate, tiles);
     hipLaunchKernelGGL(moe_grouped_down_kernel, grid_for((H + 255) / 256), dim3(256), 0, s, (bf16_t*)y_sorted,
                        (const bf16_t*)act_sorted, (const bf16_t*)down, tile_expert, H, F, tiles);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(M), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)y_sorted, slot_of_pair, wts, H, top);

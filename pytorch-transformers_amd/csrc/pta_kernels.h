@@ -14,7 +14,7 @@
 
 #include <stdint.h>
 
-#define PTA_ABI_VERSION 13
+#define PTA_ABI_VERSION 14
 
 #ifdef __cplusplus
 extern "C" {
@@ -297,6 +297,16 @@ int pta_head_norm_rope_cache(void* q_out, const void* q_in, const void* k_in, co
 
 // ---- gates between two products (gated.hip) ---------------------------------------------------------------------------
 enum PtaGlu { PTA_GLU_SILU = 0, PTA_GLU_CLAMPED = 1 };
+// How an expert's gate and up products meet: kind PTA_GLU_SILU is act(g) * u with the launch's activation; kind
+// PTA_GLU_CLAMPED is, with g' = min(g, limit) and u' = clamp(u, -limit, limit), g' * sigmoid(alpha g') * (u' + 1).
+typedef struct PtaGate {
+    int kind;
+    float alpha;
+    float limit;
+} PtaGate;
+// PolyNorm between two products: out = a N(z) + b N(z^2) + c N(z^3) + e with powers element by element, N(v) = v /
+// sqrt(mean over the row of v^2 + eps), and (a, b, c, e) the four 32-bit numbers of `coef`; sums in 32-bit.
+int pta_polynorm(void* out, const void* z, long z_ld, const float* coef, float eps, int M, int F, int dtype, void* stream);
 int pta_gated_heads(void* out, const void* x, int x_f32, long x_ld, int x_head, const void* g, long g_ld, const float* w,
                     float eps, int M, int heads, int dv, int dtype, void* stream);
 int pta_glu(void* out, const void* gate, const void* up, long in_ld, int M, int F, int kind, float alpha, float limit,
@@ -309,16 +319,29 @@ int pta_decay_scan(float* y, const void* q, const void* k, const void* v, long l
 
 // ---- routed experts (moe.hip) -----------------------------------------------------------------------------------------
 enum PtaRouteScore { PTA_ROUTE_SIGMOID = 0, PTA_ROUTE_SOFTMAX = 1 };
-int pta_moe_route(int* ids, float* wts, const void* h, long h_ld, const float* Wr, int M, int H, int E, int top,
-                  int score_kind, int normalise, float scale, int dtype, void* stream);
+int pta_moe_route(int* ids, float* wts, const void* h, long h_ld, const float* Wr, const float* br, int M, int H, int E,
+                  int top, int score_kind, int normalise, float scale, int dtype, void* stream);
 int pta_moe_up(void* act_out, const void* h, long h_ld, const void* gate_up, const int* ids, int M, int H, int F, int top,
-               int act, int dtype, void* stream);
+               int act, const PtaGate* gate_how, int dtype, void* stream);
 int pta_moe_down(void* out, const void* act_in, const void* down, const int* ids, const float* wts, int M, int H, int F,
                  int top, int dtype, void* stream);
 int pta_moe_grouped_slots(int pairs, int E);
 int pta_moe_grouped(void* out, const void* x, long x_ld, const void* gate_up, const void* down, const int* ids,
                     const float* wts, int* sorted_pair, int* slot_of_pair, int* tile_expert, void* act_sorted, void* y_sorted,
-                    int M, int H, int F, int E, int top, int act, void* stream);
+                    int M, int H, int F, int E, int top, int act, const PtaGate* gate_how, void* stream);
+
+// ---- LayerNorm around a 32-bit stream (ln_stream.hip) -------------------------------------------------------------------
+int pta_layernorm_stream(void* out_narrow, float* out_wide, const float* x, const void* y, long y_ld, const float* wy,
+                         const float* by, float mult, const float* add, const float* vec, const int* rows, const float* w,
+                         const float* b, float eps, int M, int H, int dtype, void* stream);
+// out[m] = table[ids[m]] * scale + pos_table[min(token_pos[m], positions - 1)], 32-bit (embed_norm.hip)
+int pta_embed_pos(float* out, const void* table, const int* ids, const void* pos_table, const int* token_pos, float scale,
+                  int M, int H, int positions, int dtype, void* stream);
+
+// ---- attention whose heads' scores are capped and mixed before the softmax (attn_talk.hip) -----------------------------
+int pta_attn_talk(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
+                  const int* token_seq, const int* token_pos, const float* talk, float softcap, int M, int nh, int nkv, int d,
+                  float scale, int window, int chunk, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

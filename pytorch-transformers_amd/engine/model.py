@@ -20,7 +20,7 @@ import weakref
 import numpy as np
 import torch
 
-from .. import host, tuning
+from .. import host, ops, tuning
 from ..cache.paged import PagedCache
 from ..config.registry import AutoConfig, lookup
 from ..parts.base import ResidualSum, StepContext, WideResidual, as_tensor
@@ -443,7 +443,10 @@ class CausalLM:
 
     def forward_tokens(self, ctx: StepContext, token_ids: torch.Tensor, logit_rows: Optional[torch.Tensor]):
         """Embedding, the layers in their run order, final norm and head on the wanted rows."""
-        x = self.spec.embedding.forward(token_ids)
+        embedding = self.spec.embedding
+        x = embedding.forward(token_ids, ctx) if getattr(embedding, "wants_context", False) else embedding.forward(token_ids)
+        if self.spec.keep_embedding_output:
+            ctx.extras["embedding_output"] = x if x.dtype == torch.float32 else ops.widen(x)
         blocks = self.spec.blocks
         for i, call in enumerate(self.spec.order):
             block = blocks[call.block]

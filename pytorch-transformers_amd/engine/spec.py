@@ -18,6 +18,7 @@ INT = "int"  # integer tables: int32
 INIT_NORMAL = "normal"  # N(0, std)
 INIT_ONE_NOISE = "one_noise"  # 1 + N(0, noise)   (reference: ones)
 INIT_ZERO_NOISE = "zero_noise"  # N(0, noise)     (reference: zeros)
+INIT_EYE_NOISE = "eye_noise"  # the unit matrix + N(0, noise): a square matrix that mixes its inputs a little
 
 
 @dataclasses.dataclass(frozen=True)
@@ -79,6 +80,9 @@ class LayerCall:
     #: further storage of this entry by the name its block knows it under: ``((name, cache group, layer), ...)``,
     #: for a block that keeps something per sequence beside what its mixer keeps (``also("shift")``)
     more: Tuple[Tuple[str, str, int], ...] = ()
+    #: t if pass t of a loop (a run of layers that runs several times with the same weights) starts with this entry:
+    #: a block with a ``loop_entry`` then adds the loop's terms for that pass in front of itself
+    loop_pass: Optional[int] = None
 
     def also(self, name: str) -> Tuple[str, int]:
         """(cache group, layer) of the further storage called ``name``."""
@@ -103,6 +107,8 @@ class ModelSpec:
     #: False if a part reads the step's host-side lists (``ctx.slots`` ...) while it runs: such a step
     #: cannot be captured into a graph and replayed with other values
     supports_graphs: bool = True
+    #: True: the embedding's output (32-bit) is kept for the step as ``ctx.extras["embedding_output"]``
+    keep_embedding_output: bool = False
 
     def parts(self) -> Sequence[Any]:
         out = [self.embedding, *self.blocks]

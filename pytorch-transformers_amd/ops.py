@@ -24,7 +24,7 @@ QKV_LAYOUT_CODES = {"grouped": 0, "tail": 1, "interleaved": 2}
 ACT_CODES = {None: 0, "none": 0, "linear": 0, "gelu": 1, "gelu_python": 1, "gelu_new": 2, "gelu_pytorch_tanh": 2,
              "gelu_fast": 2, "gelu_accurate": 2, "quick_gelu": 3, "relu": 4, "relu2": 5, "relu6": 6, "silu": 7, "swish": 7,
              "sigmoid": 8, "tanh": 9, "leaky_relu": 10, "mish": 11, "gelu_10": 12, "laplace": 13}
-ABI_VERSION = 13
+ABI_VERSION = 14
 PAIRING_CODES = {"half": 0, "interleaved": 1}  # PtaPairing: elements (i, i + rotary_dim / 2) or (2i, 2i + 1)
 BIAS_OF_CODES = {"key": 0, "distance": 1}  # PtaBiasOf: the slope times the key's position, or times key - query position
 
@@ -32,6 +32,10 @@ BIAS_OF_CODES = {"key": 0, "distance": 1}  # PtaBiasOf: the slope times the key'
 class _PtaRotation(ctypes.Structure):
     _fields_ = [("inv_freq", ctypes.c_void_p), ("inv_freq_ld", ctypes.c_int), ("cs_scale", ctypes.c_float),
                 ("rotary_dim", ctypes.c_int), ("pairing", ctypes.c_int)]
+
+
+class _PtaGate(ctypes.Structure):
+    _fields_ = [("kind", ctypes.c_int), ("alpha", ctypes.c_float), ("limit", ctypes.c_float)]
 
 
 class _PtaScoreBias(ctypes.Structure):
@@ -292,6 +296,84 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = 
     return out
 
 
+def embed_pos(table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0, pos_table: Optional[torch.Tensor] = None,
+              token_pos: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[m] = table[ids[m]] * scale + pos_table[token_pos[m]]`` in 32-bit: the start of a stream that is held so.
+    The caller has checked ids and positions against the tables' rows."""
+    _need(table, "table")
+    V, H = table.shape
+    _need(ids, "ids", torch.int32)
+    M = ids.numel()
+    P = 0
+    if pos_table is not None:
+        P = pos_table.shape[0]
+        _need(pos_table, "pos_table", table.dtype, (P, H))
+        _need(token_pos, "token_pos", torch.int32, (M,))
+    out = torch.empty((M, H), dtype=torch.float32, device=table.device)
+    if M:
+        _call("pta_embed_pos", _ptr(out), _ptr(table), _ptr(ids), _ptr(pos_table), _ptr(token_pos), ctypes.c_float(scale),
+              M, H, P, dtype_code(table.dtype), _stream())
+    return out
+
+
+def layernorm_stream(dtype: torch.dtype, *, x: Optional[torch.Tensor] = None, y: Optional[torch.Tensor] = None,
+                     post=None, mult: float = 1.0, add: Optional[torch.Tensor] = None, vec: Optional[torch.Tensor] = None,
+                     pre=None, eps: float = 0.0, rows: Optional[torch.Tensor] = None, want_wide: bool = True):
+    """LayerNorm around a stream held in 32-bit, one launch: ``s = x + mult * LN_post(y) + add + vec`` (each term if
+    given: ``x``, ``add`` ``[tokens, H]`` 32-bit, ``y`` ``[tokens, H]`` in ``dtype`` with rows that may lie apart, ``vec``
+    ``[H]`` 32-bit, ``post = (weight, bias)``), then ``LN_pre(s)`` in ``dtype`` if ``pre = (weight, bias)`` is given.
+    LN is ``(v - mean) / sqrt(var + eps) * weight + bias`` with the biased variance.  ``rows`` takes those rows of the
+    inputs alone.  Returns ``(narrow or None, s or None)``; s is returned only if ``want_wide``."""
+    ref = x if x is not None else y
+    if ref is None:
+        raise KernelError("layernorm_stream needs a stream or a sublayer's output")
+    H = ref.shape[1]
+    y_ld = 0
+    if x is not None:
+        _need(x, "x", torch.float32, (x.shape[0], H))
+    if y is not None:
+        y_ld = _rows_of(y, "y", H, dtype)
+        if post is None:
+            raise KernelError("a sublayer's output needs the norm that stands on it")
+        _need(post[0], "post weight", torch.float32, (H,))
+        _need(post[1], "post bias", torch.float32, (H,))
+        if x is not None and y.shape[0] != x.shape[0]:
+            raise KernelError("x and y differ in their number of rows")
+    if add is not None:
+        _need(add, "add", torch.float32, (ref.shape[0], H))
+    if vec is not None:
+        _need(vec, "vec", torch.float32, (H,))
+    if pre is not None:
+        _need(pre[0], "pre weight", torch.float32, (H,))
+        _need(pre[1], "pre bias", torch.float32, (H,))
+    if rows is not None:
+        _need(rows, "rows", torch.int32)
+        M = rows.numel()
+    else:
+        M = ref.shape[0]
+    wide = torch.empty((M, H), dtype=torch.float32, device=ref.device) if (want_wide or pre is None) else None
+    narrow = torch.empty((M, H), dtype=dtype, device=ref.device) if pre is not None else None
+    if M:
+        _call("pta_layernorm_stream", _ptr(narrow), _ptr(wide), _ptr(x), _ptr(y), ctypes.c_long(y_ld),
+              _ptr(post[0]) if y is not None else None, _ptr(post[1]) if y is not None else None, ctypes.c_float(mult),
+              _ptr(add), _ptr(vec), _ptr(rows), _ptr(pre[0]) if pre is not None else None,
+              _ptr(pre[1]) if pre is not None else None, ctypes.c_float(eps), M, H, dtype_code(dtype), _stream())
+    return narrow, wide
+
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    """``a N(z) + b N(z^2) + c N(z^3) + e`` row by row, with powers element by element, ``N(v) = v / sqrt(mean(v^2) +
+    eps)`` and ``coef = (a, b, c, e)`` 32-bit; sums in 32-bit."""
+    M, F = z.shape
+    ld = _rows_of(z, "z", F)
+    _need(coef, "coef", torch.float32, (4,))
+    out = torch.empty((M, F), dtype=z.dtype, device=z.device)
+    if M:
+        _call("pta_polynorm", _ptr(out), _ptr(z), ctypes.c_long(ld), _ptr(coef), ctypes.c_float(eps), M, F,
+              dtype_code(z.dtype), _stream())
+    return out
+
+
 def layernorm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, *, w2=None, b2=None,
               rows: Optional[torch.Tensor] = None):
     """LayerNorm of the rows of x (or of x[rows]); with (w2, b2) a second affine output of the same pass."""
@@ -459,6 +541,36 @@ def attn_generic(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_
     return out
 
 
+def attn_talk_sizes_problem(nh: int, nkv: int, d: int) -> Optional[str]:
+    """Why ``attn_talk`` does not take these sizes, or None."""
+    lib = load_library()
+    if lib.pta_attn_talk_sizes_ok(int(nh), int(nkv), int(d)):
+        return lib.pta_last_error().decode("utf-8", "replace")
+    return None
+
+
+def attn_talk(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_pos, scale: float, *,
+              talk: Optional[torch.Tensor] = None, softcap: float = 0.0, window: int = 0, chunk: int = 0):
+    """Causal attention as ``attn_generic`` (no bias) whose scores are, before the softmax, capped (``softcap *
+    tanh(score / softcap)`` if ``softcap`` > 0) and mixed over the heads (``score_h <- sum_g talk[h, g] score_g`` if
+    ``talk`` ``[nh, nh]`` 32-bit is given); 32-bit arithmetic; out [M, nh*d]."""
+    _need(q, "q")
+    M, nh, d = q.shape
+    nkv = k_pool.shape[1]
+    _need_pools(k_pool, v_pool, q.dtype, nkv, d)
+    _need(block_table, "block_table", torch.int32)
+    _need(token_seq, "token_seq", torch.int32, (M,))
+    _need(token_pos, "token_pos", torch.int32, (M,))
+    if talk is not None:
+        _need(talk, "talk", torch.float32, (nh, nh))
+    out = torch.empty((M, nh * d), dtype=q.dtype, device=q.device)
+    if M:
+        _call("pta_attn_talk", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), block_table.shape[1],
+              _ptr(token_seq), _ptr(token_pos), _ptr(talk), ctypes.c_float(softcap), M, nh, nkv, d, ctypes.c_float(scale),
+              int(window), int(chunk), dtype_code(q.dtype), _stream())
+    return out
+
+
 def gemm_f32(a: torch.Tensor, w: torch.Tensor, bias=None, act=None, add1=None, add2=None) -> torch.Tensor:
     """act(a @ w.T + bias) + add1 + add2 in true 32-bit with a fixed summation order."""
     _need(a, "a", torch.float32)
@@ -560,6 +672,14 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
                          bias_scale=bias_scale, chunk=chunk)
     return attn_generic(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, slopes, scale, window, alibi_exact,
                         bias_of, bias_scale, chunk)
+
+
+def attention_talk(q: torch.Tensor, k_pool, v_pool, block_table, ctx, scale: float, *, talk=None, softcap: float = 0.0,
+                   window: int = 0, chunk: int = 0) -> torch.Tensor:
+    """Attention of a step's tokens over the cache with capped scores that are mixed over the heads before the
+    softmax (``attn_talk``): picks the kernel for the step's shape and type."""
+    return attn_talk(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, scale, talk=talk, softcap=softcap,
+                     window=window, chunk=chunk)
 
 
 def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0,
@@ -1560,17 +1680,20 @@ ROUTE_SCORE_CODES = {"sigmoid": 0, "softmax": 1}
 
 
 def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, score: str = "sigmoid", normalise: bool = True,
-              scale: float = 1.0):
-    """Per token the ``top`` experts with the largest scores of ``router @ h`` (32-bit; ``router`` ``[experts,
-    features]`` 32-bit) and their weights: ``(ids [M, top] int32, weights [M, top] 32-bit)``."""
+              scale: float = 1.0, bias: Optional[torch.Tensor] = None):
+    """Per token the ``top`` experts with the largest scores of ``router @ h`` (+ ``bias``; 32-bit; ``router``
+    ``[experts, features]`` and ``bias`` ``[experts]`` 32-bit) and their weights: ``(ids [M, top] int32, weights [M,
+    top] 32-bit)``."""
     M, H = h.shape
     E = router.shape[0]
     _need(router, "router", torch.float32, (E, H))
+    if bias is not None:
+        _need(bias, "router bias", torch.float32, (E,))
     ld = _rows_of(h, "h", H)
     ids = torch.empty((M, top), dtype=torch.int32, device=h.device)
     wts = torch.empty((M, top), dtype=torch.float32, device=h.device)
     if M:
-        _call("pta_moe_route", _ptr(ids), _ptr(wts), _ptr(h), ctypes.c_long(ld), _ptr(router), M, H, E, int(top),
+        _call("pta_moe_route", _ptr(ids), _ptr(wts), _ptr(h), ctypes.c_long(ld), _ptr(router), _ptr(bias), M, H, E, int(top),
               ROUTE_SCORE_CODES[score], int(bool(normalise)), ctypes.c_float(scale), dtype_code(h.dtype), _stream())
     return ids, wts
 
@@ -1579,9 +1702,14 @@ MOE_GROUPED_FROM_ROWS = 16  # steps of more tokens run their experts on the matr
 
 
 def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor,
-                act: str = "silu") -> torch.Tensor:
+                act: str = "silu", gate=None) -> torch.Tensor:
     """``sum_k wts[m, k] * down[e] (act(gate[e] h) * (up[e] h))`` with ``e = ids[m, k]``: ``gate_up`` ``[experts, 2 F,
-    features]`` (an expert's gate rows, then its up rows), ``down`` ``[experts, features, F]``; out ``[M, features]``."""
+    features]`` (an expert's gate rows, then its up rows), ``down`` ``[experts, features, F]``; out ``[M, features]``.
+    ``gate = (kind, alpha, limit)`` of ``GLU_CODES``: with ``"clamped"`` an expert's two products meet as ``glu`` says
+    in place of ``act(g) * u``."""
+    how = None
+    if gate is not None:
+        how = ctypes.byref(_PtaGate(GLU_CODES[gate[0]], float(gate[1]), float(gate[2])))
     M, H = h.shape
     E, F2, _ = gate_up.shape
     F = F2 // 2
@@ -1602,12 +1730,12 @@ def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids:
         y_sorted = torch.empty((slots, H), dtype=h.dtype, device=h.device)
         _call("pta_moe_grouped", _ptr(out), _ptr(h), ctypes.c_long(ld), _ptr(gate_up), _ptr(down), _ptr(ids), _ptr(wts),
               _ptr(ints[:slots]), _ptr(ints[slots:slots + M * top]), _ptr(ints[slots + M * top:]), _ptr(act_sorted),
-              _ptr(y_sorted), M, H, F, E, top, ACT_CODES[act], _stream())
+              _ptr(y_sorted), M, H, F, E, top, ACT_CODES[act], how, _stream())
         return out
     act_buf = torch.empty((M * top, F), dtype=h.dtype, device=h.device)
     if M:
         _call("pta_moe_up", _ptr(act_buf), _ptr(h), ctypes.c_long(ld), _ptr(gate_up), _ptr(ids), M, H, F, top,
-              ACT_CODES[act], dtype_code(h.dtype), _stream())
+              ACT_CODES[act], how, dtype_code(h.dtype), _stream())
         _call("pta_moe_down", _ptr(out), _ptr(act_buf), _ptr(down), _ptr(ids), _ptr(wts), M, H, F, top,
               dtype_code(h.dtype), _stream())
     return out

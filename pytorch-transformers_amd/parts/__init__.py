@@ -4,11 +4,11 @@ from .linear import Embedding, Linear, OutputHead, QkvTail, TailDone
 from .norms import LayerNorm, RMSNorm
 from .positions import AlibiPositions, NoPositions, Rotation, RotaryPositions, ScoreBias, alibi_slopes
 from .attention import AttentionMixer
-from .feedforward import DenseFeedForward, GatedFeedForward, RoutedFeedForward
-from .blocks import ParallelBlock, PostNormBlock, SequentialBlock, ShiftedParallelBlock
+from .feedforward import DenseFeedForward, GatedFeedForward, PolyNormFeedForward, RoutedFeedForward
+from .blocks import ParallelBlock, PostNormBlock, SandwichBlock, SequentialBlock, ShiftedParallelBlock
 from .gated_attention import GatedAttentionMixer
 from .linear_attention import DecayLinearAttentionMixer
-from .depth import DepthMix
+from .depth import DepthMix, LoopEntry
 from .latent_attention import LatentAttentionMixer
 from .recurrent import GatedScanMixer, StateSpaceMixer
 
@@ -16,4 +16,5 @@ __all__ = ["Part", "StepContext", "make_part", "register_part", "registered_part
            "OutputHead", "LayerNorm", "AlibiPositions", "NoPositions", "Rotation", "RotaryPositions", "ScoreBias", "alibi_slopes",
            "AttentionMixer", "DenseFeedForward", "ParallelBlock", "SequentialBlock", "PostNormBlock", "RMSNorm", "DepthMix",
            "LatentAttentionMixer", "GatedScanMixer", "StateSpaceMixer", "GatedFeedForward", "RoutedFeedForward",
-           "ShiftedParallelBlock", "GatedAttentionMixer", "DecayLinearAttentionMixer"]
+           "ShiftedParallelBlock", "GatedAttentionMixer", "DecayLinearAttentionMixer", "SandwichBlock", "LoopEntry",
+           "PolyNormFeedForward"]

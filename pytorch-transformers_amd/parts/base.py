@@ -172,6 +172,40 @@ class WideSum(WideResidual):
         return self.wide if self.dtype == torch.float32 else self.wide.to(self.dtype)
 
 
+class PendingNormSum(WideResidual):
+    """A 32-bit stream whose last sublayer is not added yet: ``x + mult * LN(y) * weight + bias`` with ``x`` the stream
+    before the sublayer, ``y`` the sublayer's output in the compute type and ``post = (weight, bias)`` the norm that
+    stands on it (``eps`` inside its root).  The launch that reads the stream next (the next block's first norm, the
+    final norm) forms it on its way (``launch_terms`` are its arguments for ``ops.layernorm_stream``); anyone else who
+    asks for ``wide`` has it formed then."""
+
+    def __init__(self, x: torch.Tensor, y: torch.Tensor, post, mult: float, eps: float, dtype: torch.dtype):
+        self.x, self.y, self.post, self.mult, self.eps, self.dtype = x, y, post, float(mult), float(eps), dtype
+        self.history = None
+        self._wide = None
+
+    @property
+    def formed(self) -> bool:
+        return self._wide is not None
+
+    def launch_terms(self) -> Dict[str, Any]:
+        if self._wide is not None:
+            return {"x": self._wide}
+        return {"x": self.x, "y": self.y, "post": self.post, "mult": self.mult}
+
+    @property
+    def wide(self) -> torch.Tensor:
+        if self._wide is None:
+            from .. import ops
+
+            self._wide = ops.layernorm_stream(self.dtype, eps=self.eps, **self.launch_terms())[1]
+        return self._wide
+
+    @property
+    def narrow(self) -> torch.Tensor:
+        return self.wide if self.dtype == torch.float32 else self.wide.to(self.dtype)
+
+
 def as_tensor(x):
     """A tensor from what a part may hand on: a tensor, a ``PartialProduct``, a ``ResidualSum`` or a
     ``WideResidual`` (its 32-bit side)."""

@@ -18,7 +18,7 @@ from typing import Optional, Sequence
 import torch
 
 from ..engine.spec import INIT_ZERO_NOISE, VECTOR, TensorSpec
-from .base import Part, ResidualSum, StepContext, WideResidual, WideSum, as_tensor, register_part
+from .base import Part, PendingNormSum, ResidualSum, StepContext, WideResidual, WideSum, as_tensor, register_part
 from .linear import Linear, PendingProjection
 
 
@@ -251,6 +251,71 @@ class ShiftedParallelBlock(Part):
         return WideSum(stream, [mixed, ff], ctx.dtype)
 
 
+class SandwichBlock(Part):
+    """A norm in front of and behind each sublayer, over a stream kept in 32-bit:
+
+        x <- x + m * norm_mixer_out(mixer(norm_mixer(x)));   x <- x + m * norm_ffn_out(ffn(norm_ffn(x)))
+
+    with ``m`` a constant and the four norms LayerNorms with weight and bias and one eps (``ops.layernorm_stream``: the
+    norm behind a sublayer, the addition and the norm in front of the next sublayer are one launch, across the
+    block's end too: the block hands its last sublayer on not yet added, ``PendingNormSum``).  ``feed_forward`` may be
+    None (a layer of the mixer alone).  ``loop_entry`` (``parts.depth.LoopEntry``): where the run order's entry says
+    that a pass of a loop starts with this block (``call.loop_pass``), the terms that the loop adds to the stream in
+    front of the pass ride in the block's first launch."""
+
+    accepts_sum = False
+    accepts_wide = True
+
+    def __init__(self, mixer: Part, feed_forward: Optional[Part], norm_mixer: Part, norm_mixer_out: Part,
+                 norm_ffn: Optional[Part], norm_ffn_out: Optional[Part], residual_mult: float = 1.0,
+                 loop_entry: Optional[Part] = None):
+        if not ((feed_forward is None) == (norm_ffn is None) == (norm_ffn_out is None)):
+            raise ValueError("a feed-forward and its two norms come together or not at all")
+        norms = [n for n in (norm_mixer, norm_mixer_out, norm_ffn, norm_ffn_out) if n is not None]
+        if any(not hasattr(n, "affine") for n in norms) or len({n.eps for n in norms}) != 1:
+            raise ValueError("the block's launches take LayerNorms with weight and bias and one eps")
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.norm_mixer, self.norm_mixer_out, self.norm_ffn, self.norm_ffn_out = norm_mixer, norm_mixer_out, norm_ffn, norm_ffn_out
+        self.residual_mult, self.eps = float(residual_mult), norm_mixer.eps
+        self.loop_entry = loop_entry
+
+    def children(self) -> Sequence[Part]:
+        return tuple(p for p in (self.norm_mixer, self.norm_mixer_out, self.norm_ffn, self.norm_ffn_out, self.mixer,
+                                 self.feed_forward, self.loop_entry) if p is not None)
+
+    def after_load(self) -> None:
+        for part in (self.mixer, self.feed_forward):
+            if part is not None and hasattr(part, "after_load"):
+                part.after_load()
+
+    def forward(self, x, ctx: StepContext, call):
+        from .. import ops
+
+        dtype, eps, m = ctx.dtype, self.eps, self.residual_mult
+        if isinstance(x, PendingNormSum) and not x.formed and x.eps == eps:
+            terms = x.launch_terms()
+        elif isinstance(x, WideResidual):
+            terms = {"x": x.wide}
+        else:
+            x = as_tensor(x)
+            terms = {"x": x if x.dtype == torch.float32 else ops.widen(x)}
+        if self.loop_entry is not None and getattr(call, "loop_pass", None) is not None:
+            add, vec = self.loop_entry.terms(call.loop_pass, ctx)
+            terms.update(add=add, vec=vec)
+        changed = len(terms) > 1  # the launch forms a stream that is not in memory yet
+        h, wide = ops.layernorm_stream(dtype, pre=self.norm_mixer.affine(), eps=eps, want_wide=changed, **terms)
+        if not changed:
+            wide = terms["x"]
+        mixed = self.mixer.forward(h, ctx, call)
+        if self.feed_forward is None:
+            return PendingNormSum(wide, mixed, self.norm_mixer_out.affine(), m, eps, dtype)
+        h, wide = ops.layernorm_stream(dtype, x=wide, y=mixed, post=self.norm_mixer_out.affine(), mult=m,
+                                       pre=self.norm_ffn.affine(), eps=eps)
+        out = self.feed_forward.forward(h, ctx)
+        return PendingNormSum(wide, out, self.norm_ffn_out.affine(), m, eps, dtype)
+
+
+register_part("block", "sandwich", SandwichBlock)
 register_part("block", "shifted_parallel", ShiftedParallelBlock)
 register_part("block", "post_norm", PostNormBlock)
 register_part("block", "parallel", ParallelBlock)

@@ -12,7 +12,7 @@ from typing import Dict, List, Optional
 import torch
 
 from .. import ops
-from ..engine.spec import INIT_ONE_NOISE, VECTOR, TensorSpec
+from ..engine.spec import INIT_ONE_NOISE, INIT_ZERO_NOISE, VECTOR, TensorSpec
 from .base import Part, register_part
 
 
@@ -63,4 +63,36 @@ class DepthMix(Part):
         return ops.depth_mix(history.planes, self.weight, history.filled, dtype)
 
 
+class LoopEntry(Part):
+    """What a run of layers that runs ``times`` times in a row with the same weights adds to the stream in front of
+    each pass t = 0, 1, ...: the embedding's output again (in front of every pass but the first; ``again=False``:
+    never), then row t of a learned table ``[times, features]`` (``name`` is its name in the file as it stands).  The
+    model keeps the embedding's 32-bit output for the step (``ModelSpec.keep_embedding_output``) in
+    ``ctx.extras["embedding_output"]``; the block that a pass starts with adds the terms in its first launch."""
+
+    def __init__(self, name: str, times: int, features: int, again: bool = True):
+        if times < 1:
+            raise ValueError(f"{name}: a loop of {times} passes")
+        self.name, self.times, self.features, self.again = name, int(times), int(features), bool(again)
+        self.steps: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(self.name, (self.times, self.features), VECTOR, INIT_ZERO_NOISE)]
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.steps = tensors[self.name]
+
+    def terms(self, t: int, ctx):
+        """``(tensor or None, vector)`` to add in front of pass ``t``, both 32-bit."""
+        if not (0 <= t < self.times):
+            raise RuntimeError(f"{self.name}: pass {t} of {self.times}")
+        add = None
+        if self.again and t > 0:
+            add = ctx.extras.get("embedding_output")
+            if add is None:
+                raise RuntimeError(f"{self.name}: the model did not keep the embedding's output for the step")
+        return add, self.steps[t]
+
+
+register_part("stream", "loop_entry", LoopEntry)
 register_part("stream", "depth_mix", DepthMix)

@@ -9,7 +9,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from .. import ops
-from ..engine.spec import INIT_NORMAL, MATRIX, VECTOR, TensorSpec
+from ..engine.spec import INIT_NORMAL, INIT_ONE_NOISE, INIT_ZERO_NOISE, MATRIX, VECTOR, TensorSpec
 from .base import Part, StepContext, as_tensor, register_part
 from .linear import Linear, PendingProjection
 
@@ -43,6 +43,32 @@ class DenseFeedForward(Part):
         if defer:
             return PendingProjection(self.down, h)
         return self.down(h, add1=as_tensor(add1), add2=as_tensor(add2))
+
+
+class PolyNormFeedForward(Part):
+    """``down(act(up(x)))`` without biases, with the activation PolyNorm: over a token's vector z of ``ffn_size`` values,
+    ``a N(z) + b N(z^2) + c N(z^3) + e`` with powers element by element, ``N(v) = v / sqrt(mean(v^2) + eps)`` and four
+    learned numbers (a, b, c, e).  The mean squares are 32-bit.  The file holds ``name.up``, ``name.down`` and the four
+    numbers as ``name.act``."""
+
+    def __init__(self, name: str, hidden_size: int, ffn_size: int, eps: float):
+        self.name, self.eps, self.ffn_size = name, float(eps), int(ffn_size)
+        self.up = Linear(f"{name}.up", hidden_size, ffn_size, False, weight_name=f"{name}.up")
+        self.down = Linear(f"{name}.down", ffn_size, hidden_size, False, weight_name=f"{name}.down")
+        self.coef: Optional[torch.Tensor] = None
+
+    def children(self) -> Sequence[Part]:
+        return (self.up, self.down)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(f"{self.name}.act", (4,), VECTOR, INIT_ONE_NOISE)]
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.coef = tensors[f"{self.name}.act"]
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None):
+        y = ops.polynorm(self.up(x), self.coef, self.eps)
+        return self.down(y, add1=as_tensor(add1), add2=as_tensor(add2))
 
 
 class GatedFeedForward(Part):
@@ -106,12 +132,18 @@ class RoutedFeedForward(Part):
         weight_e = s_e / (sum of the taken s + 1e-20) * scale     (``normalise=False``: s_e * scale)
         out = sum over the taken e of weight_e * down_e(act(gate_e x) * up_e(x))
 
+    ``router_bias``: z has a learned bias added (``name.router.b`` in the file).  ``gate = (kind, alpha, limit)``: an
+    expert's two input products meet as ``ops.glu`` of that kind says (``"clamped"``: ``g = min(gate, limit)``, ``u =
+    clamp(up, -limit, limit)``, ``g * sigmoid(alpha g) * (u + 1)``) in place of ``act(gate) * up``.
+
     The file holds ``name.router`` ``[experts, hidden]`` and per expert ``name.e<j>.gate``, ``.up`` ``[ff, hidden]``
     and ``.down`` ``[hidden, ff]``; on the device the experts' matrices are stacked (gate rows then up rows per
     expert, and the down matrices) and the router is 32-bit."""
 
     def __init__(self, name: str, hidden_size: int, ffn_size: int, experts: int, top: int, scale: float = 1.0,
-                 score: str = "sigmoid", normalise: bool = True, act: str = "silu"):
+                 score: str = "sigmoid", normalise: bool = True, act: str = "silu", router_bias: bool = False, gate=None):
+        if gate is not None and gate[0] not in ops.GLU_CODES:
+            raise ValueError(f"{name}: a gate of kind {gate[0]!r} is not built; built: {sorted(ops.GLU_CODES)}")
         if not (0 < top <= experts):
             raise ValueError(f"{name}: {top} of {experts} experts per token")
         if score not in ops.ROUTE_SCORE_CODES:
@@ -119,13 +151,15 @@ class RoutedFeedForward(Part):
         self.name, self.hidden_size, self.ffn_size = name, int(hidden_size), int(ffn_size)
         self.experts, self.top, self.scale = int(experts), int(top), float(scale)
         self.score, self.normalise, self.act = score, bool(normalise), act
-        self.router = self.gate_up = self.down = None
+        self.router_bias, self.gate = bool(router_bias), (None if gate is None else (gate[0], float(gate[1]), float(gate[2])))
+        self.router = self.gate_up = self.down = self.bias = None
 
     def tensor_specs(self) -> List[TensorSpec]:
         n, E, F, H = self.name, self.experts, self.ffn_size, self.hidden_size
         gu = tuple((f"{n}.e{e}.{m}", (F, H)) for e in range(E) for m in ("gate", "up"))
         dn = tuple((f"{n}.e{e}.down", (H, F)) for e in range(E))
-        return [TensorSpec(f"{n}.router", (E, H), VECTOR, INIT_NORMAL),
+        bias = [TensorSpec(f"{n}.router.b", (E,), VECTOR, INIT_ZERO_NOISE)] if self.router_bias else []
+        return bias + [TensorSpec(f"{n}.router", (E, H), VECTOR, INIT_NORMAL),
                 TensorSpec(f"{n}.experts.gate_up", (E, 2 * F, H), MATRIX, INIT_NORMAL, pieces=gu,
                            assemble=_stack_experts(E, (F, F)), split=_unstack_experts((F, F))),
                 TensorSpec(f"{n}.experts.down", (E, H, F), MATRIX, INIT_NORMAL, pieces=dn, assemble=_stack_experts(E, (H,)),
@@ -134,14 +168,15 @@ class RoutedFeedForward(Part):
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         n = self.name
         self.router, self.gate_up, self.down = tensors[f"{n}.router"], tensors[f"{n}.experts.gate_up"], tensors[f"{n}.experts.down"]
+        self.bias = tensors[f"{n}.router.b"] if self.router_bias else None
 
     def check_sizes(self) -> None:
         if self.top > 64 or self.experts > 2048:
             raise ValueError(f"{self.name}: the router takes at most 64 of at most 2048 experts")
 
     def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None):
-        ids, wts = ops.moe_route(x, self.router, self.top, self.score, self.normalise, self.scale)
-        out = ops.moe_experts(x, self.gate_up, self.down, ids, wts, self.act)
+        ids, wts = ops.moe_route(x, self.router, self.top, self.score, self.normalise, self.scale, bias=self.bias)
+        out = ops.moe_experts(x, self.gate_up, self.down, ids, wts, self.act, gate=self.gate)
         if add1 is None and add2 is None:
             return out
         return ops.epilogue_(out, None, None, as_tensor(add1), as_tensor(add2))
@@ -149,4 +184,5 @@ class RoutedFeedForward(Part):
 
 register_part("feed_forward", "dense", DenseFeedForward)
 register_part("feed_forward", "gated", GatedFeedForward)
+register_part("feed_forward", "polynorm", PolyNormFeedForward)
 register_part("feed_forward", "routed", RoutedFeedForward)

@@ -7,7 +7,10 @@ With h the mixer's input, H query heads on G key/value heads, queries and keys o
     q, k <- head / sqrt(mean(head^2) + eps) * w_q | w_k    one weight [key_dim] for all heads, before the rotation
     q, k <- rotated by position                            (``positions``: any rotation the kernels take)
     v    <- head / sqrt(mean(head^2) + eps)                no weight; cached so
-    score(i, j) = q_i . k_j * scale, softmax over the keys j <= i that i sees:
+    score(i, j) = q_i . k_j * scale
+    score <- softcap * tanh(score / softcap)               (``softcap`` > 0)
+    score_h <- sum_g T[h, g] score_g                       (``talk``: a learned [H, H] matrix mixes the heads' scores)
+    softmax over the keys j <= i that i sees:
         all of them, those of i's own block of ``chunk`` positions (blocks counted from the sequence's start),
         and / or the last ``window``
     out = W_o (heads side by side * sigmoid(W_g h))
@@ -23,7 +26,7 @@ from typing import Dict, List, Optional, Sequence
 import torch
 
 from .. import ops
-from ..engine.spec import INIT_ONE_NOISE, VECTOR, TensorSpec
+from ..engine.spec import INIT_EYE_NOISE, INIT_ONE_NOISE, VECTOR, TensorSpec
 from .base import Part, StepContext, register_part
 from .linear import Linear
 from .positions import as_rotation
@@ -39,7 +42,7 @@ def attention_frame(key_dim: int, value_dim: int) -> int:
 class GatedAttentionMixer(Part):
     def __init__(self, name: str, hidden_size: int, num_heads: int, kv_heads: int, key_dim: int, value_dim: int,
                  scale: float, eps: float, positions: Part, chunk: int = 0, window: int = 0, qk_norm: bool = True,
-                 v_norm: bool = True, gate: bool = True):
+                 v_norm: bool = True, gate: bool = True, softcap: float = 0.0, talk: bool = False):
         if num_heads % kv_heads:
             raise ValueError(f"{name}: heads ({num_heads}) must be a multiple of kv heads ({kv_heads})")
         self.name, self.hidden_size = name, int(hidden_size)
@@ -47,6 +50,8 @@ class GatedAttentionMixer(Part):
         self.scale, self.eps, self.positions = float(scale), float(eps), positions
         self.chunk, self.window = int(chunk), int(window)
         self.qk_norm, self.v_norm, self.gate = bool(qk_norm), bool(v_norm), bool(gate)
+        self.softcap, self.talk = float(softcap), bool(talk)
+        self.talk_w: Optional[torch.Tensor] = None
         self.frame = attention_frame(key_dim, value_dim)
         bare = lambda short, i, o: Linear(f"{name}.{short}", i, o, False, weight_name=f"{name}.{short}")
         self.q = bare("q", hidden_size, self.num_heads * self.key_dim)
@@ -61,14 +66,19 @@ class GatedAttentionMixer(Part):
         return tuple(p for p in (self.q, self.k, self.v, self.g, self.out, self.positions) if p is not None)
 
     def tensor_specs(self) -> List[TensorSpec]:
-        if not self.qk_norm:
-            return []
-        return [TensorSpec(f"{self.name}.q.norm", (self.key_dim,), VECTOR, INIT_ONE_NOISE),
-                TensorSpec(f"{self.name}.k.norm", (self.key_dim,), VECTOR, INIT_ONE_NOISE)]
+        specs = []
+        if self.qk_norm:
+            specs += [TensorSpec(f"{self.name}.q.norm", (self.key_dim,), VECTOR, INIT_ONE_NOISE),
+                      TensorSpec(f"{self.name}.k.norm", (self.key_dim,), VECTOR, INIT_ONE_NOISE)]
+        if self.talk:
+            specs.append(TensorSpec(f"{self.name}.talk", (self.num_heads, self.num_heads), VECTOR, INIT_EYE_NOISE))
+        return specs
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         if self.qk_norm:
             self.q_w, self.k_w = tensors[f"{self.name}.q.norm"], tensors[f"{self.name}.k.norm"]
+        if self.talk:
+            self.talk_w = tensors[f"{self.name}.talk"]
 
     def after_load(self) -> None:
         self.inp = Linear.stacked(f"{self.name}.qkvg", [p for p in (self.q, self.k, self.v, self.g) if p is not None])
@@ -80,8 +90,10 @@ class GatedAttentionMixer(Part):
             problem = f"heads of {max(self.key_dim, self.value_dim)} elements are more than the 256 the kernels take"
         if problem is None and rot is not None:
             problem = ops.rotation_problem(self.key_dim, rot.rotary_dim, rot.pairing)
-        if problem is None and (self.chunk < 0 or self.window < 0):
-            problem = "chunk and window are 0 (none) or positive"
+        if problem is None and (self.chunk < 0 or self.window < 0 or self.softcap < 0):
+            problem = "chunk, window and softcap are 0 (none) or positive"
+        if problem is None and (self.talk or self.softcap):
+            problem = ops.attn_talk_sizes_problem(self.num_heads, self.kv_heads, self.frame)
         if problem is not None:
             raise ValueError(f"{self.name}: {problem}")
 
@@ -99,7 +111,11 @@ class GatedAttentionMixer(Part):
         q = ops.head_norm_rope_cache(proj[:, at[0]:at[1]], proj[:, at[1]:at[2]], proj[:, at[2]:at[3]], self.q_w, self.k_w,
                                      self.eps, self.v_norm, as_rotation(self.positions.rotation()), ctx, table, k_pool,
                                      v_pool, H, G, dk, dv, write_cache=call.write_cache)
-        o = ops.attention(q, k_pool, v_pool, table, ctx, None, self.scale, self.window, chunk=self.chunk)
+        if self.talk or self.softcap:
+            o = ops.attention_talk(q, k_pool, v_pool, table, ctx, self.scale, talk=self.talk_w, softcap=self.softcap,
+                                   window=self.window, chunk=self.chunk)
+        else:
+            o = ops.attention(q, k_pool, v_pool, table, ctx, None, self.scale, self.window, chunk=self.chunk)
         if self.gate:
             o = ops.gated_heads(o, self.frame, proj[:, at[3]:], H, dv, x.dtype)
         elif self.frame != dv:

@@ -241,23 +241,46 @@ class PendingProjection:
 
 
 class Embedding(Part):
-    """``h[t] = E[id_t]``, no scaling (src/transformers/models/falcon/modeling_falcon.py:835, :895-896)."""
+    """``h[t] = E[id_t]``, no scaling (src/transformers/models/falcon/modeling_falcon.py:835, :895-896).
 
-    def __init__(self, name: str, vocab_size: int, hidden_size: int, weight_name: Optional[str] = None):
+    With ``scale`` and / or ``position_name`` (a learned table ``[max_positions, hidden]`` under that name in the file):
+    ``h[t] = E[id_t] * scale + P[position of t]``, formed and handed on in 32-bit as the start of a stream that is held
+    so; the model then calls ``forward(ids, ctx)`` (``wants_context``)."""
+
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, weight_name: Optional[str] = None, scale: float = 1.0,
+                 position_name: Optional[str] = None, max_positions: int = 0):
         self.name = name
         self.weight_name = weight_name or name + ".weight"
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
+        self.scale, self.position_name, self.max_positions = float(scale), position_name, int(max_positions)
+        if position_name is not None and self.max_positions <= 0:
+            raise ValueError(f"{name}: a position table needs its number of positions")
+        self.wants_context = position_name is not None or self.scale != 1.0
         self.weight: Optional[torch.Tensor] = None
+        self.positions: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [TensorSpec(self.weight_name, (self.vocab_size, self.hidden_size), MATRIX, INIT_NORMAL)]
+        specs = [TensorSpec(self.weight_name, (self.vocab_size, self.hidden_size), MATRIX, INIT_NORMAL)]
+        if self.position_name is not None:
+            specs.append(TensorSpec(self.position_name, (self.max_positions, self.hidden_size), MATRIX, INIT_NORMAL))
+        return specs
 
     def load(self, tensors) -> None:
         self.weight = tensors[self.weight_name]
+        if self.position_name is not None:
+            self.positions = tensors[self.position_name]
 
-    def forward(self, ids: torch.Tensor) -> torch.Tensor:
-        return ops.embed(self.weight, ids)
+    def forward(self, ids: torch.Tensor, ctx=None) -> torch.Tensor:
+        if not self.wants_context:
+            return ops.embed(self.weight, ids)
+        if self.positions is not None and ctx.starts and ctx.new_tokens:
+            # (a replayed step has no host lists: the step that was launched directly before it was checked here)
+            longest = max(s + n for s, n in zip(ctx.starts, ctx.new_tokens))
+            if longest > self.max_positions:
+                raise ValueError(f"{self.name}: a sequence of {longest} tokens is longer than the {self.max_positions} "
+                                 "positions the model has vectors for")
+        return ops.embed_pos(self.weight, ids, self.scale, self.positions, ctx.token_pos if self.positions is not None else None)
 
 
 class OutputHead(Part):
@@ -265,9 +288,12 @@ class OutputHead(Part):
     (src/transformers/models/falcon/modeling_falcon.py:1163-1168, :1230; the reference casts the
     rows it samples from to 32-bit, src/transformers/generation/utils.py:3247)."""
 
-    def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str], scale: float = 1.0):
-        """``scale``: a factor on the logits (applied to the 32-bit result)."""
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str], scale: float = 1.0,
+                 weight_name: Optional[str] = None):
+        """``scale``: a factor on the logits (applied to the 32-bit result).  ``weight_name``: the matrix's name in
+        the file as it stands (default ``name.weight``)."""
         self.name = name
+        self.weight_name = weight_name or name + ".weight"
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.tied_to = tied_to
@@ -275,11 +301,11 @@ class OutputHead(Part):
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [TensorSpec(self.name + ".weight", (self.vocab_size, self.hidden_size), MATRIX, INIT_NORMAL,
+        return [TensorSpec(self.weight_name, (self.vocab_size, self.hidden_size), MATRIX, INIT_NORMAL,
                            tied_to=self.tied_to)]
 
     def load(self, tensors) -> None:
-        self.weight = tensors[self.name + ".weight"]
+        self.weight = tensors[self.weight_name]
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         return ops.scale_(self._product(h), self.scale)

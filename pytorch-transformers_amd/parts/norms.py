@@ -12,20 +12,39 @@ from .base import Part, ResidualSum, register_part
 
 
 class LayerNorm(Part):
-    def __init__(self, name: str, hidden_size: int, eps: float):
+    def __init__(self, name: str, hidden_size: int, eps: float, weight_name: Optional[str] = None,
+                 bias_name: Optional[str] = None):
+        """``weight_name``, ``bias_name``: the two vectors' names in the file as they stand (default ``name.weight``,
+        ``name.bias``)."""
         self.name = name
         self.hidden_size = hidden_size
         self.eps = float(eps)
+        self.weight_name, self.bias_name = weight_name or name + ".weight", bias_name or name + ".bias"
         self.weight: Optional[torch.Tensor] = None
         self.bias: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [TensorSpec(self.name + ".weight", (self.hidden_size,), VECTOR, INIT_ONE_NOISE),
-                TensorSpec(self.name + ".bias", (self.hidden_size,), VECTOR, INIT_ZERO_NOISE)]
+        return [TensorSpec(self.weight_name, (self.hidden_size,), VECTOR, INIT_ONE_NOISE),
+                TensorSpec(self.bias_name, (self.hidden_size,), VECTOR, INIT_ZERO_NOISE)]
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.weight = tensors[self.name + ".weight"]
-        self.bias = tensors[self.name + ".bias"]
+        self.weight = tensors[self.weight_name]
+        self.bias = tensors[self.bias_name]
+
+    def affine(self):
+        """(weight, bias), for a launch that applies this norm beside other work (``ops.layernorm_stream``)."""
+        return self.weight, self.bias
+
+    def forward_wide(self, x, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The norm of a stream held in 32-bit (a ``WideResidual``), in its compute type.  A stream whose last
+        sublayer is still to be normed and added (``PendingNormSum``) has that done in the same launch."""
+        from .base import PendingNormSum
+
+        dtype = getattr(x, "dtype", None) or x.narrow.dtype
+        if isinstance(x, PendingNormSum) and not x.formed and x.eps == self.eps:
+            return ops.layernorm_stream(dtype, pre=self.affine(), eps=self.eps, rows=rows, want_wide=False,
+                                        **x.launch_terms())[0]
+        return ops.layernorm_stream(dtype, x=x.wide, pre=self.affine(), eps=self.eps, rows=rows, want_wide=False)[0]
 
     def _wide_loads(self, x: torch.Tensor) -> bool:
         # bfloat16 rows of a width the sixteen-byte kernel takes: the one that also forms residual sums

@@ -16,7 +16,7 @@ from typing import Dict, Optional, Sequence
 
 import torch
 
-from ..engine.spec import INIT_NORMAL, INIT_ONE_NOISE, INIT_ZERO_NOISE, INT, TensorSpec
+from ..engine.spec import INIT_EYE_NOISE, INIT_NORMAL, INIT_ONE_NOISE, INIT_ZERO_NOISE, INT, TensorSpec
 from .loader import device_dtype_for, save_weights
 
 
@@ -40,6 +40,10 @@ def init_tensor(spec: TensorSpec, seed: int, std: float, *, noise: Optional[floa
         t.normal_(0.0, noise, generator=g).add_(1.0)
     elif spec.init == INIT_ZERO_NOISE:
         t.normal_(0.0, noise, generator=g)
+    elif spec.init == INIT_EYE_NOISE:
+        if len(spec.shape) != 2 or spec.shape[0] != spec.shape[1]:
+            raise ValueError(f"{spec.name}: a unit matrix with noise is square, not {spec.shape}")
+        t.normal_(0.0, noise, generator=g).add_(torch.eye(spec.shape[0], dtype=torch.float32, device=device))
     else:
         raise ValueError(f"{spec.name}: unknown init {spec.init!r}")
     return t.to(dtype)
