@@ -119,7 +119,7 @@ class GatedAttentionMixer(Part):
         if self.gate:
             o = ops.gated_heads(o, self.frame, proj[:, at[3]:], H, dv, x.dtype)
         elif self.frame != dv:
-            o = o.view(-1, H, self.frame)[:, :, :dv].reshape(-1, H * dv)
+            o = o.view(-1, H, self.frame)[:, :, :dv].reshape(-1, H * dv).contiguous()
         return self.out(o, add1=residual)
 
 
