@@ -436,6 +436,40 @@ def bimepel_config(size, layers, vocab=32768):
                          norm={"eps": 1e-6}, initializer_range=0.02)
 
 
+# ---- the Kekapel design beside the same Falcon model (--design kekapel) --------------------------------------------------
+KEKAPEL_SIZES = {
+    # width; the dense feed-forward (two matrices, as Falcon's); attention heads of 128 on 8 KV heads over a window of
+    # 1,024 positions, scores capped at 30 and mixed over the heads; 16 experts of three matrices of which a token uses 2,
+    # which together are as large as the dense feed-forward
+    "2k": dict(width=2048, ff=8192, heads=16, expert_ff=2752),
+    "4k": dict(width=4096, ff=16384, heads=32, expert_ff=5440),
+}
+KEKAPEL_WINDOW = 1024
+KEKAPEL_KERNEL_LABELS = {
+    "pta_layernorm_stream": "LayerNorm behind a sublayer, addition into the 32-bit stream, LayerNorm in front of the next",
+    "pta_embed_pos": "scaled embedding plus position vector",
+    "pta_polynorm": "PolyNorm between the dense feed-forward's two products",
+    "pta_attn_talk": "attention with capped scores mixed over the heads, 32-bit kernel (a token's heads in one workgroup)",
+    "pta_attn_talk_mfma": "attention with capped scores mixed over the heads, matrix cores (prompts)",
+}
+
+
+def kekapel_config(size, layers, vocab=32768):
+    """Four layers (dense, experts, dense, experts feed-forward) of which the middle two run ``layers - 2`` / 2 times:
+    ``layers`` layer runs."""
+    from pytorch_transformers_amd import KekapelConfig
+
+    z = KEKAPEL_SIZES[size]
+    dense = {"kind": "dense", "ff": z["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": z["expert_ff"], "limit": 7.0}, "router": {"experts": 16, "top": 2}}
+    attn = {"heads": z["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0,
+            "mask": {"size": KEKAPEL_WINDOW}}
+    kinds = [{"type": "attention", "mixer": attn, "mlp": m} for m in (dense, moe, dense, moe)]
+    return KekapelConfig(vocab=vocab, width=z["width"], max_positions=8192, embedding={"scale": 1.0}, layers=kinds,
+                         loop={"start": 1, "stop": 3, "times": max(1, (layers - 2) // 2)}, norm={"eps": 1e-5},
+                         residual_mult=0.7, initializer_range=0.02)
+
+
 def falcon_like(size, layers, vocab=32768):
     """The closest model the library had: Falcon's new architecture at the same width, feed-forward, depth and
     vocabulary, heads of 128 in 8 groups."""
@@ -459,8 +493,9 @@ def design_record(args):
     ops.load_library()
     KERNEL_LABELS.update(PAVODRA_KERNEL_LABELS)
     KERNEL_LABELS.update(BIMEPEL_KERNEL_LABELS)
+    KERNEL_LABELS.update(KEKAPEL_KERNEL_LABELS)
     design = args.design
-    design_config = pavodra_config if design == "pavodra" else bimepel_config
+    design_config = {"pavodra": pavodra_config, "bimepel": bimepel_config, "kekapel": kekapel_config}[design]
     gen_cfg = GenerationConfig(do_sample=False, eos_token_id=None)
     layers, T, ctx_len = args.layers or 6, args.prefill_tokens, args.prompt_len
     out = {"design": design, "beside": "falcon (new architecture, 8 KV groups of head size 128)", "dtype": args.dtype,
@@ -494,6 +529,12 @@ def design_record(args):
                     kv = b * (ctx_len % block + 1) * a["kv_heads"] * (a["dim"] + a["vdim"]) * 2
                     seen = sum(min(block, T - s0) * (min(block, T - s0) + 1) / 2 for s0 in range(0, T, block))
                     fl = 2.0 * (a["dim"] + a["vdim"]) * a["heads"] * seen
+                elif name == "kekapel":  # the keys and values inside a token's window only
+                    a = cfg.layers[0]["mixer"]
+                    win = a["mask"]["size"]
+                    kv = b * min(win, ctx_len + 1) * a["kv_heads"] * (a["dim"] + a["vdim"]) * 2
+                    seen = sum(min(win, t + 1) for t in range(T))
+                    fl = 2.0 * (a["dim"] + a["vdim"]) * a["heads"] * seen
                 else:
                     kv = b * (ctx_len + 1) * 2 * cfg.kv_heads * cfg.head_dim * 2
                     fl = 2.0 * cfg.head_dim * cfg.num_attention_heads * T * (T + 1)
@@ -521,7 +562,7 @@ def design_record(args):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", default=None, choices=["pavodra", "bimepel"],
+    ap.add_argument("--design", default=None, choices=["pavodra", "bimepel", "kekapel"],
                     help="measure that design beside the closest Falcon model at equal layer sizes and print that record "
                          "instead of the default run's (--layers, --prefill-tokens, --prompt-len and --dtype apply)")
     ap.add_argument("--design-sizes", default="2k,4k", help="with --design: which of the layer sizes 2k, 4k")

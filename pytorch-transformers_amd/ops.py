@@ -174,7 +174,8 @@ def _entry_cost(name: str, a) -> tuple:
         return gemm(a[6], a[7], a[8], 4)
     if name == "pta_layernorm_sum":
         return ((a[4] + a[7]) * float(a[17]) * a[19] * 4, 0.0)
-    if name in ("pta_attn_mfma", "pta_attn_generic", "pta_attn_latent_mfma", "pta_attn_latent"):
+    if name in ("pta_attn_mfma", "pta_attn_generic", "pta_attn_latent_mfma", "pta_attn_latent", "pta_attn_talk",
+                "pta_attn_talk_mfma"):
         return (float(timing_hint.get("attn_bytes", 0)), float(timing_hint.get("attn_flops", 0)))
     val = lambda i: float(getattr(a[i], "value", a[i]) or 0)
     given = lambda i: 1.0 if getattr(a[i], "value", a[i]) else 0.0
@@ -216,9 +217,16 @@ def _entry_cost(name: str, a) -> tuple:
         M, heads, P, N, e = float(timing_hint.get("rows", 0)), a[12], a[13], a[14], el(a[18])
         return (M * heads * ((2 * N + P) * e + P * 4.0), 4.0 * M * heads * N * P)
     if name == "pta_moe_route":
-        return (float(a[5]) * a[6] * el(a[12]) + float(a[6]) * a[7] * 4.0, 2.0 * a[5] * a[6] * a[7])
+        return (float(a[6]) * a[7] * el(a[13]) + float(a[7]) * a[8] * 4.0, 2.0 * a[6] * a[7] * a[8])
+    if name == "pta_layernorm_stream":  # what it reads and writes: the stream, a sublayer's output, a second tensor, the results
+        M, H, e = float(a[14]), float(a[15]), el(a[16])
+        return (M * H * ((given(2) + given(8) + given(1)) * 4.0 + (given(3) + given(0)) * e), 0.0)
+    if name == "pta_polynorm":
+        return (float(a[5]) * a[6] * 2.0 * el(a[7]), 0.0)
+    if name == "pta_embed_pos":
+        return (float(a[6]) * a[7] * (2.0 * el(a[9]) + 4.0), 0.0)
     if name == "pta_moe_up":  # at most every (token, expert) pair's matrices once, and no more than all experts'
-        M, H, Fe, top, e = float(a[5]), a[6], a[7], a[8], el(a[10])
+        M, H, Fe, top, e = float(a[5]), a[6], a[7], a[8], el(a[11])
         pairs = min(M * top, float(timing_hint.get("experts", M * top)))
         return (pairs * 2 * Fe * H * e, 4.0 * M * top * Fe * H)
     if name == "pta_moe_down":
