@@ -84,6 +84,21 @@ __global__ __launch_bounds__(64 * WAVES) void attn_combine_kernel(bf16_t* __rest
     }
 }
 
+extern "C" int pta_attn_combine(void* out, const float* po, const float* pm, const float* pl, long n_rows, int d,
+                                int n_splits, void* stream) {
+    PTA_REQUIRE(n_rows > 0 && n_rows <= 0x7fffffffL && d > 0 && d <= 256 && d % 4 == 0 && n_splits >= 1,
+                "attn_combine: %ld rows of %d elements in %d ranges", n_rows, d, n_splits);
+    hipStream_t s = (hipStream_t)stream;
+    int lps = 4;  // lanes that share a split's vector of d floats, a float4 each
+    while (lps * 4 < d) lps *= 2;
+    const dim3 rows((unsigned)n_rows);
+    if (n_splits > 4 * (64 / lps))  // more splits than one wave has in flight at once
+        hipLaunchKernelGGL(attn_combine_kernel<4>, rows, dim3(256), 0, s, (bf16_t*)out, po, pm, pl, d, n_splits, lps);
+    else
+        hipLaunchKernelGGL(attn_combine_kernel<1>, rows, dim3(64), 0, s, (bf16_t*)out, po, pm, pl, d, n_splits, lps);
+    return pta_check_launch("attn_combine");
+}
+
 extern "C" int pta_attn_decode_shared_ok(int d, int heads_per_kv_head) {
     return d % 16 == 0 && heads_per_kv_head > 0 && decode_shared_built(d / 16, (heads_per_kv_head + 15) / 16);
 }
@@ -188,15 +203,6 @@ extern "C" int pta_attn_mfma(void* out, const void* q, const void* k_pool, const
 #undef PTA_ATTN_CASE
     int rc = pta_check_launch("attn_mfma");
     if (rc) return rc;
-    if (n_splits > 1) {
-        int lps = 4;  // lanes that share a split's vector of d floats, a float4 each
-        while (lps * 4 < d) lps *= 2;
-        const dim3 rows((unsigned)((long)M * nh));
-        if (n_splits > 4 * (64 / lps))  // more splits than one wave has in flight at once
-            hipLaunchKernelGGL(attn_combine_kernel<4>, rows, dim3(256), 0, s, (bf16_t*)out, po, pm, pl, d, n_splits, lps);
-        else
-            hipLaunchKernelGGL(attn_combine_kernel<1>, rows, dim3(64), 0, s, (bf16_t*)out, po, pm, pl, d, n_splits, lps);
-        rc = pta_check_launch("attn_combine");
-    }
+    if (n_splits > 1) rc = pta_attn_combine(out, po, pm, pl, (long)M * nh, d, n_splits, stream);
     return rc;
 }

@@ -1,0 +1,55 @@
+// The entry point of the attention with capped, mixed scores on the matrix cores; the kernel and its launchers are in
+// attn_talk_mfma_impl.h, instantiated per head size in attn_talk_mfma_dt*.hip.
+#include "attn_talk_mfma_impl.h"
+
+#define PTA_TALK_HEAD(DT_) extern template bool talk_launch_head<DT_>(const TalkLaunch&, int);
+PTA_TALK_HEAD(1) PTA_TALK_HEAD(2) PTA_TALK_HEAD(3) PTA_TALK_HEAD(4) PTA_TALK_HEAD(5) PTA_TALK_HEAD(6) PTA_TALK_HEAD(7)
+PTA_TALK_HEAD(8)
+#undef PTA_TALK_HEAD
+
+// heads a wave holds: as many as the head size allows, all of one KV head, with at most sixteen waves; 0: none fits
+static int talk_heads_per_wave(int nh, int nkv, int d) {
+    if (nh <= 0 || nkv <= 0 || nh % nkv || d % 16 || d < 16 || d > 128) return 0;
+    if ((size_t)nh * 4096 > 128 * 1024) return 0;  // the heads' tiles of two blocks of keys in LDS
+    const int g = nh / nkv;
+    for (int ct = talk_max_heads(d / 16); ct >= 1; ct /= 2)
+        if (g % ct == 0 && nh / ct <= 16) return ct;
+    return 0;
+}
+
+extern "C" int pta_attn_talk_mfma_supported(int nh, int nkv, int d) { return talk_heads_per_wave(nh, nkv, d) > 0; }
+
+extern "C" int pta_attn_talk_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
+                                  int bt_stride, const int* cu_tokens, const int* seq_start, const float* talk, float softcap,
+                                  int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int window, int chunk,
+                                  int split_size, int n_splits, float* po, float* pm, float* pl, void* stream) {
+    PTA_REQUIRE(n_seqs > 0 && max_new > 0 && M > 0, "attn_talk_mfma: sizes must be positive");
+    const int ct = talk_heads_per_wave(nh, nkv, d);
+    PTA_REQUIRE(ct > 0, "attn_talk_mfma: %d heads on %d KV heads of size %d are not built (sizes 16..128 in steps of 16, "
+                "at most 32 heads, at most 16 groups of heads that fit a wave)", nh, nkv, d);
+    PTA_REQUIRE(window >= 0 && chunk >= 0 && softcap >= 0.f, "attn_talk_mfma: window, chunk and softcap are 0 (none) or positive");
+    PTA_REQUIRE(n_splits >= 1 && n_splits <= 1024, "attn_talk_mfma: n_splits must be 1..1024, got %d", n_splits);
+    PTA_REQUIRE(n_splits == 1 || (max_new == 1 && split_size > 0 && split_size % 64 == 0 && po && pm && pl),
+                "attn_talk_mfma: ranges of keys are for one token per sequence, with a size that is a multiple of 64 and "
+                "buffers for the partial results");
+    PTA_REQUIRE((long)n_seqs * n_splits <= 65535, "attn_talk_mfma: too many sequences x ranges for one launch");
+    PTA_REQUIRE(out && q && k_pool && v_pool && block_table && cu_tokens && seq_start, "attn_talk_mfma: null pointer");
+    PTA_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pool % 16) == 0 && ((uintptr_t)v_pool % 16) == 0 &&
+                    ((uintptr_t)out % 8) == 0, "attn_talk_mfma: pointers must be 16-byte aligned");
+    // cap * tanh(s scale / cap) is evaluated as cap - 2 cap / (1 + 2^(s pre_mul))
+    const float pre_mul = softcap > 0.f ? 2.0f * scale * TALK_LOG2E / softcap : scale;
+    const TalkLaunch a{(bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table,
+                       bt_stride, cu_tokens, seq_start, talk, softcap, pre_mul, n_seqs, max_new, nh, nkv, window, chunk,
+                       split_size, n_splits, (hipStream_t)stream};
+    bool built = false;
+    switch (d / 16) {
+#define PTA_TALK_CASE(DT_) case DT_: built = talk_launch_head<DT_>(a, ct); break;
+        PTA_TALK_CASE(1) PTA_TALK_CASE(2) PTA_TALK_CASE(3) PTA_TALK_CASE(4) PTA_TALK_CASE(5) PTA_TALK_CASE(6)
+        PTA_TALK_CASE(7) PTA_TALK_CASE(8)
+#undef PTA_TALK_CASE
+    }
+    if (!built) return pta_fail("attn_talk_mfma: no kernel for %d heads a wave at head size %d", ct, d);
+    int rc = pta_check_launch("attn_talk_mfma");
+    if (rc || n_splits == 1) return rc;
+    return pta_attn_combine(out, po, pm, pl, (long)M * nh, d, n_splits, stream);
+}

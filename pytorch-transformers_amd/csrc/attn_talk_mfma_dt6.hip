@@ -1,0 +1,4 @@
+// The attention with mixed heads on the matrix cores for heads of 96 elements (see attn_talk_mfma_impl.h).
+#include "attn_talk_mfma_impl.h"
+
+template bool talk_launch_head<6>(const TalkLaunch&, int);

@@ -342,6 +342,17 @@ int pta_embed_pos(float* out, const void* table, const int* ids, const void* pos
 int pta_attn_talk(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
                   const int* token_seq, const int* token_pos, const float* talk, float softcap, int M, int nh, int nkv, int d,
                   float scale, int window, int chunk, int dtype, void* stream);
+// The same on the matrix cores (bfloat16; attn_talk_mfma.hip): a step's tokens by sequence (cu_tokens, seq_start) as
+// pta_attn_mfma takes them; with one token per sequence the keys may be cut into n_splits ranges of split_size.
+int pta_attn_talk_mfma_supported(int nh, int nkv, int d);
+int pta_attn_talk_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
+                       int bt_stride, const int* cu_tokens, const int* seq_start, const float* talk, float softcap,
+                       int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int window, int chunk,
+                       int split_size, int n_splits, float* po, float* pm, float* pl, void* stream);
+// Merge of the partial results of ranges of keys (attn_mfma.hip): out[row] = sum_s w_s po[row, s] / sum_s w_s pl[row, s],
+// w_s = 2^(pm[row, s] - max_s pm); a range whose pm is -inf is not read.
+int pta_attn_combine(void* out, const float* po, const float* pm, const float* pl, long rows, int d, int n_splits,
+                     void* stream);
 
 #ifdef __cplusplus
 }

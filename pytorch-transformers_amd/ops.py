@@ -682,10 +682,67 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
                         bias_of, bias_scale, chunk)
 
 
+def attn_talk_mfma_ok(q: torch.Tensor, nkv: int) -> bool:
+    """Whether the matrix-core kernel for capped, mixed scores takes these queries (bfloat16, sizes built)."""
+    return q.dtype == torch.bfloat16 and bool(
+        load_library().pta_attn_talk_mfma_supported(int(q.shape[1]), int(nkv), int(q.shape[2])))
+
+
+def attn_talk_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start, scale: float, *, max_new: int,
+                   talk: Optional[torch.Tensor] = None, softcap: float = 0.0, window: int = 0, chunk: int = 0,
+                   n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS) -> torch.Tensor:
+    """``attn_talk`` on the matrix cores (bfloat16 in, 32-bit scores, mix and softmax); out [M, nh*d].  ``max_new``
+    bounds the new tokens of any sequence of the step; with one token per sequence and ``n_splits`` > 1 the keys are
+    cut into ranges of ``split_size`` (``n_splits * split_size`` bounds every context), merged by a second launch."""
+    _need(q, "q", torch.bfloat16)
+    M, nh, d = q.shape
+    nkv = k_pool.shape[1]
+    _need_pools(k_pool, v_pool, q.dtype, nkv, d)
+    _need(block_table, "block_table", torch.int32)
+    n_seqs = block_table.shape[0]
+    _need(cu_tokens, "cu_tokens", torch.int32, (n_seqs + 1,))
+    _need(seq_start, "seq_start", torch.int32, (n_seqs,))
+    if talk is not None:
+        _need(talk, "talk", torch.float32, (nh, nh))
+    out = torch.empty((M, nh * d), dtype=q.dtype, device=q.device)
+    po = pm = pl = None
+    if n_splits > 1:
+        po = torch.empty((M, nh, n_splits, d), dtype=torch.float32, device=q.device)
+        pm = torch.empty((M, nh, n_splits), dtype=torch.float32, device=q.device)
+        pl = torch.empty((M, nh, n_splits), dtype=torch.float32, device=q.device)
+    _call("pta_attn_talk_mfma", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), block_table.shape[1],
+          _ptr(cu_tokens), _ptr(seq_start), _ptr(talk), ctypes.c_float(softcap), n_seqs, int(max_new), M, nh, nkv, d,
+          ctypes.c_float(scale), int(window), int(chunk), int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl),
+          _stream())
+    return out
+
+
+def talk_decode_ranges(n_seqs: int, max_len: int, window: int = 0, chunk: int = 0) -> tuple:
+    """(ranges, keys a range) into which a decode step of ``attn_talk_mfma`` cuts the keys: about two workgroups for
+    every compute unit over the keys that a token sees at most, ranges of whole pages, at most 1,024 of them."""
+    seen = max_len
+    for bound in (window, chunk):
+        if bound > 0:
+            seen = min(seen, bound + 63)
+    wanted = max(1, min((seen + 63) // 64, -(-512 // max(n_seqs, 1))))
+    size = (-(-seen // wanted) + 63) // 64 * 64
+    size = max(size, (-(-max_len // 1024) + 63) // 64 * 64)
+    return -(-max_len // size), size
+
+
 def attention_talk(q: torch.Tensor, k_pool, v_pool, block_table, ctx, scale: float, *, talk=None, softcap: float = 0.0,
                    window: int = 0, chunk: int = 0) -> torch.Tensor:
     """Attention of a step's tokens over the cache with capped scores that are mixed over the heads before the
-    softmax (``attn_talk``): picks the kernel for the step's shape and type."""
+    softmax: picks the kernel for the step's shape and type.  bfloat16 with sizes the matrix-core kernel is built
+    for: that kernel, with the context cut into ranges when every sequence brings one token; anything else: the
+    32-bit kernel."""
+    if attn_talk_mfma_ok(q, k_pool.shape[1]):
+        n_splits, size = 1, ATTN_SPLIT_KEYS
+        if ctx.is_decode:
+            n_splits, size = talk_decode_ranges(ctx.n_seqs, ctx.max_len, window, chunk)
+        return attn_talk_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, scale,
+                              max_new=max(ctx.new_tokens), talk=talk, softcap=softcap, window=window, chunk=chunk,
+                              n_splits=n_splits, split_size=size)
     return attn_talk(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, scale, talk=talk, softcap=softcap,
                      window=window, chunk=chunk)
 

@@ -1109,6 +1109,140 @@ def test_attn_mfma_decode_shared_keys_refusals():
             _attn_case(ops, _mfma(ops, None, 0, ops.SHARED_KEYS), torch.bfloat16, nh, nkv, d, starts=[5], news=[1])
 
 
+def _talk_plain(q, k, v, scale, cap, talk, window, chunk):
+    """Attention whose scores are capped and then mixed over the heads, 64-bit: q [T, nh, d], k, v [T, nkv, d]."""
+    T, nh, d = q.shape
+    g = nh // k.shape[1]
+    t = torch.arange(T)
+    seen = t[None, :] <= t[:, None]
+    if window:
+        seen &= t[None, :] > t[:, None] - window
+    if chunk:
+        seen &= (t[None, :] // chunk) == (t[:, None] // chunk)
+    s = torch.stack([q[:, h] @ k[:, h // g].T * scale for h in range(nh)])   # [nh, T, T]
+    if cap:
+        s = cap * torch.tanh(s / cap)
+    if talk is not None:
+        s = torch.einsum("hg,gij->hij", talk.double(), s)
+    w = torch.softmax(s.masked_fill(~seen[None], float("-inf")), dim=-1)
+    return torch.stack([w[h] @ v[:, h // g] for h in range(nh)], dim=1).reshape(T, nh * d)
+
+
+def _talk_case(ops, nh, nkv, d, starts, news, cap=0.0, mix=True, window=0, chunk=0, seed=0, loud=None, ranges=None):
+    """A cache of random keys and values (NaN where nothing was written, and in pages behind every window), the new
+    tokens through ``attn_talk_mfma`` and through the 32-bit kernel, both against the plain computation.  ``loud``:
+    per sequence a key that every head's last query scores far above the others (or None)."""
+    dtype = torch.bfloat16
+    lens = [s + n for s, n in zip(starts, news)]
+    n_pages = sum((L + 63) // 64 for L in lens) + 3
+    k_pool, v_pool, bt, lists = _cache_setup(len(lens), lens, nkv, d, dtype, n_pages=n_pages, seed=seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    talk = None
+    if mix:
+        talk = (torch.eye(nh) + 0.3 * torch.randn(nh, nh, generator=g)).float()
+    scale = 1.7 / math.sqrt(d)
+    ks, vs, qs = [], [], []
+    for i, L in enumerate(lens):
+        k = torch.randn(L, nkv, d, generator=g).to(dtype)
+        v = torch.randn(L, nkv, d, generator=g).to(dtype)
+        q = torch.randn(news[i], nh, d, generator=g).to(dtype)
+        if loud is not None and loud[i] is not None:
+            k[loud[i]] = 0
+            k[loud[i], :, 0] = 6.0
+            q[-1] = 0
+            q[-1, :, 0] = 6.0 * math.sqrt(d)
+        ks.append(k); vs.append(v); qs.append(q)
+        behind = max(starts[i] - window + 1, 0) if window else 0
+        if chunk:
+            behind = max(behind, starts[i] // chunk * chunk)
+        for p, page in enumerate(lists[i]):
+            n = min(64, L - p * 64)
+            if (p + 1) * 64 <= behind:
+                continue  # no new token sees this page: it may be gone
+            k_pool[page, :, :n] = k[p * 64:p * 64 + n].transpose(0, 1).cuda()
+            v_pool[page, :, :, :n] = v[p * 64:p * 64 + n].permute(1, 2, 0).cuda()
+    q_all = torch.cat(qs).cuda()
+    token_seq = torch.tensor([i for i, n in enumerate(news) for _ in range(n)], dtype=torch.int32).cuda()
+    token_pos = torch.tensor([s + j for s, n in zip(starts, news) for j in range(n)], dtype=torch.int32).cuda()
+    cu = torch.tensor([0] + list(torch.tensor(news).cumsum(0)), dtype=torch.int32).cuda()
+    seq_start = torch.tensor(starts, dtype=torch.int32).cuda()
+    t_dev = talk.cuda() if mix else None
+    kw = {}
+    if ranges is not None:
+        kw = {"n_splits": (max(lens) + ranges - 1) // ranges, "split_size": ranges}
+    got = ops.attn_talk_mfma(q_all, k_pool, v_pool, bt, cu, seq_start, scale, max_new=max(news), talk=t_dev, softcap=cap,
+                             window=window, chunk=chunk, **kw)
+    slow = ops.attn_talk(q_all, k_pool, v_pool, bt, token_seq, token_pos, scale, talk=t_dev, softcap=cap, window=window,
+                         chunk=chunk)
+    at = 0
+    for i, (s0, n) in enumerate(zip(starts, news)):
+        L = lens[i]
+        q_full = torch.zeros(L, nh, d, dtype=torch.float64)
+        q_full[s0:] = qs[i].double()
+        want = _talk_plain(q_full, ks[i].double(), vs[i].double(), scale, cap, talk, window, chunk)[s0:]
+        for name, res in (("matrix cores", got), ("32-bit", slow)):
+            err = float((res[at:at + n].double().cpu() - want).abs().max())
+            assert err <= 2e-2 * max(1.0, float(want.abs().max())), f"{name}: sequence {i} (start {s0}, {n} new): {err:.3e}"
+        if loud is not None and loud[i] is not None and (mix is False):
+            far = vs[i][loud[i]].double().repeat_interleave(nh // nkv, 0).reshape(-1)
+            assert float((got[at + n - 1].double().cpu() - far).abs().max()) < 0.05, "the loud key does not dominate"
+        at += n
+
+
+TALK_SHAPES = [(8, 4, 48), (16, 8, 128), (4, 4, 64), (6, 2, 32), (3, 1, 16), (32, 8, 128), (16, 2, 64), (12, 12, 80),
+               (10, 2, 96), (2, 1, 112)]
+
+
+@pytest.mark.parametrize("nh,nkv,d", TALK_SHAPES)
+def test_attn_talk_mfma_prompts_and_portions(nh, nkv, d):
+    """Whole prompts, single tokens and portions over an existing cache in one launch; a cap, a mix, both, neither;
+    windows and blocks whose edges fall inside a tile of sixteen tokens and inside a block of 32 keys."""
+    ops = _ops()
+    assert ops.attn_talk_mfma_ok(torch.empty(1, nh, d, dtype=torch.bfloat16).cuda(), nkv)
+    starts, news = [0, 63, 200, 0, 127, 31], [70, 1, 5, 1, 2, 40]
+    _talk_case(ops, nh, nkv, d, starts, news, cap=5.0)
+    _talk_case(ops, nh, nkv, d, starts, news, cap=0.0, seed=1)
+    _talk_case(ops, nh, nkv, d, starts, news, cap=0.0, mix=False, seed=2, loud=[3, 40, 100, 0, None, 70])
+    _talk_case(ops, nh, nkv, d, starts, news, cap=2.0, mix=False, seed=3)
+    for window in (1, 33, 72):
+        _talk_case(ops, nh, nkv, d, starts, news, cap=4.0, window=window, seed=4)
+    _talk_case(ops, nh, nkv, d, starts, news, cap=4.0, chunk=48, seed=5)
+
+
+@pytest.mark.parametrize("nh,nkv,d", [(8, 4, 48), (16, 8, 128), (32, 8, 128), (16, 2, 64)])
+def test_attn_talk_mfma_long_prompts(nh, nkv, d):
+    """A prompt of 700 tokens and 300 new tokens over 900 cached ones: many blocks of keys per workgroup, with and
+    without a window."""
+    ops = _ops()
+    _talk_case(ops, nh, nkv, d, [0, 900, 3], [700, 300, 61], cap=6.0)
+    _talk_case(ops, nh, nkv, d, [0, 900, 3], [700, 300, 61], cap=6.0, window=200, seed=2)
+
+
+@pytest.mark.parametrize("nh,nkv,d", TALK_SHAPES)
+@pytest.mark.parametrize("ranges", [None, 64, 256])
+def test_attn_talk_mfma_decode_ranges(nh, nkv, d, ranges):
+    """One token per sequence over contexts of very different lengths, the keys whole and cut into ranges that are
+    merged; ranges before a window and past a sequence's end; a loud far key."""
+    ops = _ops()
+    starts = [0, 63, 64, 700, 255, 256, 1, 1500]
+    _talk_case(ops, nh, nkv, d, starts, [1] * 8, cap=5.0, ranges=ranges)
+    _talk_case(ops, nh, nkv, d, starts, [1] * 8, cap=0.0, mix=False, ranges=ranges, loud=[0, 5, 64, 13, None, 255, None, 1203])
+    for window in (33, 100):
+        _talk_case(ops, nh, nkv, d, starts, [1] * 8, cap=5.0, window=window, ranges=ranges, seed=window)
+    _talk_case(ops, nh, nkv, d, starts, [1] * 8, chunk=96, ranges=ranges, seed=9)
+
+
+def test_attn_talk_mfma_sizes():
+    ops = _ops()
+    lib = ops.load_library()
+    assert lib.pta_attn_talk_mfma_supported(16, 8, 128) and lib.pta_attn_talk_mfma_supported(32, 8, 128)
+    assert not lib.pta_attn_talk_mfma_supported(8, 4, 40) and not lib.pta_attn_talk_mfma_supported(8, 4, 256)
+    assert not lib.pta_attn_talk_mfma_supported(34, 34, 64) and not lib.pta_attn_talk_mfma_supported(64, 8, 64)
+    for n, length, window in ((1, 1, 0), (8, 1025, 1024), (64, 5000, 0), (3, 300000, 0), (512, 100, 72), (1, 70000, 1024)):
+        ranges, size = ops.talk_decode_ranges(n, length, window)
+        assert size % 64 == 0 and 1 <= ranges <= 1024 and ranges * size >= length
+
+
 def test_decode_plan():
     """The cut of a decode launch: whole tiles within what the head size allows, a range size that is a
     multiple of the page, the same for every batch and context of one captured step's bucket."""
