@@ -450,7 +450,7 @@ KEKAPEL_KERNEL_LABELS = {
     "pta_embed_pos": "scaled embedding plus position vector",
     "pta_polynorm": "PolyNorm between the dense feed-forward's two products",
     "pta_attn_talk": "attention with capped scores mixed over the heads, 32-bit kernel (a token's heads in one workgroup)",
-    "pta_attn_talk_mfma": "attention with capped scores mixed over the heads, matrix cores (prompts)",
+    "pta_attn_talk_mfma": "attention with capped scores mixed over the heads, matrix cores (+ merge of key ranges)",
 }
 
 
