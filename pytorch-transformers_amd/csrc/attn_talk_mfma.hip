@@ -2,6 +2,8 @@
 // attn_talk_mfma_impl.h, instantiated per head size in attn_talk_mfma_dt*.hip.
 #include "attn_talk_mfma_impl.h"
 
+#include <algorithm>
+
 #define PTA_TALK_HEAD(DT_) extern template bool talk_launch_head<DT_>(const TalkLaunch&, int);
 PTA_TALK_HEAD(1) PTA_TALK_HEAD(2) PTA_TALK_HEAD(3) PTA_TALK_HEAD(4) PTA_TALK_HEAD(5) PTA_TALK_HEAD(6) PTA_TALK_HEAD(7)
 PTA_TALK_HEAD(8)
@@ -17,6 +19,14 @@ static int talk_heads_per_wave(int nh, int nkv, int d) {
     return 0;
 }
 
+// Into how many runs a prompt launch cuts every tile's keys: the tiles alone should not leave compute units idle, a
+// run is at least four blocks of keys, and at most four partial results a row are written and merged.
+extern "C" int pta_attn_talk_prompt_ranges(int tiles, int keys_seen) {
+    const int units = pta_compute_units();
+    if (tiles <= 0 || tiles >= units) return 1;
+    return std::max(1, std::min({4, units / tiles, keys_seen / 128}));
+}
+
 extern "C" int pta_attn_talk_mfma_supported(int nh, int nkv, int d) { return talk_heads_per_wave(nh, nkv, d) > 0; }
 
 extern "C" int pta_attn_talk_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
@@ -29,9 +39,9 @@ extern "C" int pta_attn_talk_mfma(void* out, const void* q, const void* k_pool, 
                 "at most 32 heads, at most 16 groups of heads that fit a wave)", nh, nkv, d);
     PTA_REQUIRE(window >= 0 && chunk >= 0 && softcap >= 0.f, "attn_talk_mfma: window, chunk and softcap are 0 (none) or positive");
     PTA_REQUIRE(n_splits >= 1 && n_splits <= 1024, "attn_talk_mfma: n_splits must be 1..1024, got %d", n_splits);
-    PTA_REQUIRE(n_splits == 1 || (max_new == 1 && split_size > 0 && split_size % 64 == 0 && po && pm && pl),
-                "attn_talk_mfma: ranges of keys are for one token per sequence, with a size that is a multiple of 64 and "
-                "buffers for the partial results");
+    PTA_REQUIRE(n_splits == 1 || (split_size >= 0 && split_size % 64 == 0 && po && pm && pl),
+                "attn_talk_mfma: ranges of keys have a size that is a multiple of 64 (0: equal runs of every tile's "
+                "blocks) and buffers for the partial results");
     PTA_REQUIRE((long)n_seqs * n_splits <= 65535, "attn_talk_mfma: too many sequences x ranges for one launch");
     PTA_REQUIRE(out && q && k_pool && v_pool && block_table && cu_tokens && seq_start, "attn_talk_mfma: null pointer");
     PTA_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k_pool % 16) == 0 && ((uintptr_t)v_pool % 16) == 0 &&

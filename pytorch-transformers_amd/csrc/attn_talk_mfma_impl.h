@@ -17,8 +17,13 @@
 // token's result does not depend on how a prompt was cut into steps or on the batch beyond the rounding of the
 // running maximum's reference point.
 //
-// With one token per sequence the keys may be cut into ranges (split_size keys each, a workgroup per range); each
-// writes unnormalised sums with their maximum and weight sum, and pta_attn_combine merges them in range order.
+// The keys may be cut into ranges, a workgroup per range: with one token per sequence ranges of split_size keys of
+// the context; for prompts (split_size 0) every tile's own span of keys in n_splits equal runs of blocks, for launches
+// that would otherwise leave compute units idle.  Each range writes unnormalised sums with their maximum and weight
+// sum, and pta_attn_combine merges them in range order.
+//
+// The keys of the next block are asked for as soon as the products with the current ones are done, the values of the
+// current block at its start: both arrive behind the cap, the mix and the softmax of the block.
 #pragma once
 
 #include "common.h"
@@ -52,7 +57,7 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
     const int* __restrict__ seq_start, const float* __restrict__ talk, float cap, float pre_mul, int nh, int nkv,
     int window, int chunk, int split_size, int n_splits) {
     constexpr int D = DT * 16, DS = (DT + 1) / 2, CHUNKS = D / 8;
-    extern __shared__ __attribute__((aligned(16))) float4 talk_tiles[];  // [2][nh][2][64]
+    extern __shared__ __attribute__((aligned(16))) float4 talk_tiles[];  // [2][nh][2][64], then the mix [nh][nh]
     auto lowest_key = [&](int t) {
         int lo = window > 0 ? max(0, t - window + 1) : 0;
         if (chunk > 0) lo = max(lo, t / chunk * chunk);
@@ -71,8 +76,17 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
     const int first_pos = start + tok0, last_pos = start + min(tok0 + 15, n_new - 1);
     const int kv_len = start + n_new;
     const int lo_last = lowest_key(last_pos);
-    const int k_begin = max(lowest_key(first_pos) & ~31, n_splits > 1 ? split * split_size : 0);
-    const int k_end = n_splits > 1 ? min(last_pos + 1, (split + 1) * split_size) : last_pos + 1;
+    int k_begin = lowest_key(first_pos) & ~31, k_end = last_pos + 1;
+    if (n_splits > 1) {
+        if (split_size > 0) {  // ranges of the context
+            k_begin = max(k_begin, split * split_size);
+            k_end = min(k_end, (split + 1) * split_size);
+        } else {               // equal runs of this tile's blocks
+            const int per = ((k_end - k_begin + 31) / 32 + n_splits - 1) / n_splits * 32;
+            k_begin += split * per;
+            k_end = min(k_end, k_begin + per);
+        }
+    }
     const int min_lim = min(first_pos + 1, k_end);  // below this key no column masks anything for being late
 
     if (k_begin >= k_end) {  // a range that none of the tokens sees: only its marker is written
@@ -113,21 +127,37 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
     ones.u = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);
     const int* bt = block_table + (long)seq * bt_stride;
     const float cap2 = -2.0f * cap;
+    float* mix_s = reinterpret_cast<float*>(talk_tiles + (size_t)nh * 256);
+    if (talk) {
+        for (int i = threadIdx.x; i < nh * nh; i += blockDim.x) mix_s[i] = talk[i];
+        // (read only behind the first block's barrier)
+    }
+    const float* mix_row = mix_s + h0 * nh;
+
+    // key rows: tile tt, row r holds key 8*(r/4) + 4*tt + r%4 of the block, so that a lane's eight scores are
+    // those of the eight consecutive keys 8*gq .. 8*gq+7, which is what the second product's operand wants
+    TalkFrag kf[2][DS];
+    auto load_keys = [&](int kb) {
+        const long page = ((long)bt[kb >> 6] * nkv + kvh) * (long)(PTA_PAGE * D);
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+            const bf16_t* kp = k_pool + page + (long)((kb & 63) + 8 * (c >> 2) + 4 * tt + (c & 3)) * D;
+#pragma unroll
+            for (int ds = 0; ds < DS; ++ds)
+                kf[tt][ds].u = *reinterpret_cast<const uint4*>(kp + min(ds * 4 + gq, CHUNKS - 1) * 8);
+        }
+    };
+    const int kb_last = (kv_len - 1) & ~31;  // the last block that has a page
+    // (not where sixteen waves of large heads leave a wave no registers for it)
+    constexpr bool AHEAD = MAXW <= 8 || DT <= 4;
+    if constexpr (AHEAD) load_keys(k_begin);
 
     int it = 0;
     for (int kb = k_begin; kb < k_end; kb += 32, ++it) {
         const long page = ((long)bt[kb >> 6] * nkv + kvh) * (long)(PTA_PAGE * D);
         const int in_page = kb & 63;
-        // key rows: tile tt, row r holds key 8*(r/4) + 4*tt + r%4 of the block, so that a lane's eight scores are
-        // those of the eight consecutive keys 8*gq .. 8*gq+7, which is what the second product's operand wants
-        TalkFrag kf[2][DS], vf[DT];
-#pragma unroll
-        for (int tt = 0; tt < 2; ++tt) {
-            const bf16_t* kp = k_pool + page + (long)(in_page + 8 * (c >> 2) + 4 * tt + (c & 3)) * D;
-#pragma unroll
-            for (int ds = 0; ds < DS; ++ds)
-                kf[tt][ds].u = *reinterpret_cast<const uint4*>(kp + min(ds * 4 + gq, CHUNKS - 1) * 8);
-        }
+        TalkFrag vf[DT];
+        if constexpr (!AHEAD) load_keys(kb);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
             vf[dt].u = *reinterpret_cast<const uint4*>(v_pool + page + (long)(dt * 16 + c) * PTA_PAGE + in_page + gq * 8);
@@ -141,15 +171,20 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
 #pragma unroll
                 for (int ds = 0; ds < DS; ++ds)
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[tt][ds].v, qf[ct][ds].v, acc, 0, 0, 0);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float x = acc[e] * pre_mul;
-                    // cap * tanh(z) = cap - 2 cap / (1 + e^(2z)); pre_mul carries 2 scale log2(e) / cap
-                    if (cap > 0.f) x = __builtin_fmaf(cap2, __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x)), cap);
-                    acc[e] = x;
-                }
                 s[tt][ct] = acc;
             }
+        if constexpr (AHEAD) load_keys(min(kb + 32, kb_last));  // the next block's (the last one's again behind it)
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float x = s[tt][ct][e] * pre_mul;
+                    // cap * tanh(z) = cap - 2 cap / (1 + e^(2z)); pre_mul carries 2 scale log2(e) / cap
+                    if (cap > 0.f) x = __builtin_fmaf(cap2, __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x)), cap);
+                    s[tt][ct][e] = x;
+                }
 
         if (talk) {
             float4* tiles = talk_tiles + (size_t)(it & 1) * nh * 128;
@@ -164,11 +199,12 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
                 s[0][ct] = talk_f32x4_t{0.f, 0.f, 0.f, 0.f};
                 s[1][ct] = talk_f32x4_t{0.f, 0.f, 0.f, 0.f};
             }
+#pragma unroll 4
             for (int h = 0; h < nh; ++h) {
                 const float4 a0 = tiles[(h * 2) * 64 + lane], a1 = tiles[(h * 2 + 1) * 64 + lane];
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) {
-                    const float t = talk[(h0 + ct) * nh + h];
+                    const float t = mix_row[ct * nh + h];
                     s[0][ct][0] = __builtin_fmaf(t, a0.x, s[0][ct][0]); s[0][ct][1] = __builtin_fmaf(t, a0.y, s[0][ct][1]);
                     s[0][ct][2] = __builtin_fmaf(t, a0.z, s[0][ct][2]); s[0][ct][3] = __builtin_fmaf(t, a0.w, s[0][ct][3]);
                     s[1][ct][0] = __builtin_fmaf(t, a1.x, s[1][ct][0]); s[1][ct][1] = __builtin_fmaf(t, a1.y, s[1][ct][1]);
@@ -281,13 +317,13 @@ constexpr int talk_max_heads(int dt) { return dt <= 4 ? 4 : 2; }
 template <int DT, int CT, int MAXW>
 static void talk_launch_one(const TalkLaunch& a) {
     auto kern = attn_talk_mfma_kernel<DT, CT, MAXW>;
-    const size_t lds = a.talk ? (size_t)a.nh * 4096 : 0;
+    const size_t lds = a.talk ? (size_t)a.nh * 4096 + (size_t)a.nh * a.nh * 4 : 0;
     if (lds > 64 * 1024) {  // more than a launch may ask for unless the kernel has been told, once per device
         static bool told[64] = {};
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
         if (!told[dev]) {
-            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+            (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 136 * 1024);
             told[dev] = true;
         }
     }

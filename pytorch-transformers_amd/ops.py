@@ -693,7 +693,8 @@ def attn_talk_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_
                    n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS) -> torch.Tensor:
     """``attn_talk`` on the matrix cores (bfloat16 in, 32-bit scores, mix and softmax); out [M, nh*d].  ``max_new``
     bounds the new tokens of any sequence of the step; with one token per sequence and ``n_splits`` > 1 the keys are
-    cut into ranges of ``split_size`` (``n_splits * split_size`` bounds every context), merged by a second launch."""
+    cut into ranges of ``split_size`` (``n_splits * split_size`` bounds every context), merged by a second launch;
+    ``split_size`` 0: every tile of sixteen tokens cuts the keys it sees into ``n_splits`` equal runs (prompts)."""
     _need(q, "q", torch.bfloat16)
     M, nh, d = q.shape
     nkv = k_pool.shape[1]
@@ -740,6 +741,10 @@ def attention_talk(q: torch.Tensor, k_pool, v_pool, block_table, ctx, scale: flo
         n_splits, size = 1, ATTN_SPLIT_KEYS
         if ctx.is_decode:
             n_splits, size = talk_decode_ranges(ctx.n_seqs, ctx.max_len, window, chunk)
+        else:  # few tiles of sixteen tokens: each cuts its keys into runs, so that no compute unit idles
+            seen = min([ctx.max_len] + [b + 15 for b in (window, chunk) if b > 0])
+            tiles = sum((n + 15) // 16 for n in ctx.new_tokens)
+            n_splits, size = int(load_library().pta_attn_talk_prompt_ranges(tiles, seen)), 0
         return attn_talk_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, scale,
                               max_new=max(ctx.new_tokens), talk=talk, softcap=softcap, window=window, chunk=chunk,
                               n_splits=n_splits, split_size=size)

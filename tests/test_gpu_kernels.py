@@ -1168,7 +1168,9 @@ def _talk_case(ops, nh, nkv, d, starts, news, cap=0.0, mix=True, window=0, chunk
     seq_start = torch.tensor(starts, dtype=torch.int32).cuda()
     t_dev = talk.cuda() if mix else None
     kw = {}
-    if ranges is not None:
+    if ranges is not None and ranges < 0:  # every tile's keys in so many runs
+        kw = {"n_splits": -ranges, "split_size": 0}
+    elif ranges is not None:
         kw = {"n_splits": (max(lens) + ranges - 1) // ranges, "split_size": ranges}
     got = ops.attn_talk_mfma(q_all, k_pool, v_pool, bt, cu, seq_start, scale, max_new=max(news), talk=t_dev, softcap=cap,
                              window=window, chunk=chunk, **kw)
@@ -1207,6 +1209,9 @@ def test_attn_talk_mfma_prompts_and_portions(nh, nkv, d):
     for window in (1, 33, 72):
         _talk_case(ops, nh, nkv, d, starts, news, cap=4.0, window=window, seed=4)
     _talk_case(ops, nh, nkv, d, starts, news, cap=4.0, chunk=48, seed=5)
+    for runs in (2, 3, 4):  # more runs than some tiles have blocks of keys
+        _talk_case(ops, nh, nkv, d, starts, news, cap=5.0, seed=6, ranges=-runs)
+        _talk_case(ops, nh, nkv, d, starts, news, cap=5.0, window=72, seed=7, ranges=-runs)
 
 
 @pytest.mark.parametrize("nh,nkv,d", [(8, 4, 48), (16, 8, 128), (32, 8, 128), (16, 2, 64)])
@@ -1216,6 +1221,8 @@ def test_attn_talk_mfma_long_prompts(nh, nkv, d):
     ops = _ops()
     _talk_case(ops, nh, nkv, d, [0, 900, 3], [700, 300, 61], cap=6.0)
     _talk_case(ops, nh, nkv, d, [0, 900, 3], [700, 300, 61], cap=6.0, window=200, seed=2)
+    _talk_case(ops, nh, nkv, d, [0, 900, 3], [700, 300, 61], cap=6.0, seed=3, ranges=-3)
+    _talk_case(ops, nh, nkv, d, [0, 900, 3], [700, 300, 61], cap=6.0, window=200, seed=4, ranges=-2)
 
 
 @pytest.mark.parametrize("nh,nkv,d", TALK_SHAPES)
@@ -1238,6 +1245,8 @@ def test_attn_talk_mfma_sizes():
     assert lib.pta_attn_talk_mfma_supported(16, 8, 128) and lib.pta_attn_talk_mfma_supported(32, 8, 128)
     assert not lib.pta_attn_talk_mfma_supported(8, 4, 40) and not lib.pta_attn_talk_mfma_supported(8, 4, 256)
     assert not lib.pta_attn_talk_mfma_supported(34, 34, 64) and not lib.pta_attn_talk_mfma_supported(64, 8, 64)
+    assert lib.pta_attn_talk_prompt_ranges(128, 2048) in (1, 2) and lib.pta_attn_talk_prompt_ranges(4096, 2048) == 1
+    assert lib.pta_attn_talk_prompt_ranges(4, 100) == 1 and lib.pta_attn_talk_prompt_ranges(8, 5000) == 4
     for n, length, window in ((1, 1, 0), (8, 1025, 1024), (64, 5000, 0), (3, 300000, 0), (512, 100, 72), (1, 70000, 1024)):
         ranges, size = ops.talk_decode_ranges(n, length, window)
         assert size % 64 == 0 and 1 <= ranges <= 1024 and ranges * size >= length
