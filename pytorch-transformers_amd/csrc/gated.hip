@@ -118,13 +118,67 @@ __global__ __launch_bounds__(256) void polynorm_kernel(T* __restrict__ out, cons
     }
 }
 
+// The same for bfloat16 rows whose length is a multiple of eight and that start at multiples of 16 bytes: eight
+// elements a load, long rows on 1,024 threads.
+__device__ __forceinline__ void polynorm_unpack(const uint4& u, float (&v)[8]) {
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        v[2 * j] = __uint_as_float(w[j] << 16);
+        v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    }
+}
+
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void polynorm_vec_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ z,
+                                                               long z_ld, const float* __restrict__ coef, float eps, int F) {
+    __shared__ float red[16];
+    const uint4* zr = reinterpret_cast<const uint4*>(z + (long)blockIdx.x * z_ld);
+    const int n = F / 8;
+    float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    for (int i = threadIdx.x; i < n; i += THREADS) {
+        float v[8];
+        polynorm_unpack(zr[i], v);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float v2 = v[j] * v[j];
+            s1 += v2;
+            s2 += v2 * v2;
+            s3 += v2 * v2 * v2;
+        }
+    }
+    const float inv_f = 1.0f / (float)F;
+    const float r1 = coef[0] / sqrtf(block_sum(s1, red) * inv_f + eps);
+    const float r2 = coef[1] / sqrtf(block_sum(s2, red) * inv_f + eps);
+    const float r3 = coef[2] / sqrtf(block_sum(s3, red) * inv_f + eps);
+    const float e = coef[3];
+    uint4* orow = reinterpret_cast<uint4*>(out + (long)blockIdx.x * F);
+    for (int i = threadIdx.x; i < n; i += THREADS) {
+        float v[8];
+        polynorm_unpack(zr[i], v);
+        bf16_t r[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float v2 = v[j] * v[j];
+            r[j] = f32_to_bf16_bits(r1 * v[j] + r2 * v2 + r3 * (v2 * v[j]) + e);
+        }
+        orow[i] = *reinterpret_cast<const uint4*>(r);
+    }
+}
+
 extern "C" int pta_polynorm(void* out, const void* z, long z_ld, const float* coef, float eps, int M, int F, int dtype,
                             void* stream) {
     PTA_REQUIRE(M > 0 && F > 0 && out && z && coef && z_ld >= F, "polynorm: sizes must be positive and pointers given");
     hipStream_t s = (hipStream_t)stream;
     if (dtype == PTA_F32)
         hipLaunchKernelGGL(polynorm_kernel<float>, dim3(M), dim3(256), 0, s, (float*)out, (const float*)z, z_ld, coef, eps, F);
-    else if (dtype == PTA_BF16)
+    else if (dtype == PTA_BF16 && F % 8 == 0 && z_ld % 8 == 0 && (uintptr_t)z % 16 == 0 && (uintptr_t)out % 16 == 0) {
+        // (the threads of a row follow from its length alone, so the sums' order does not depend on the batch)
+        if (F >= 8192)
+            hipLaunchKernelGGL(polynorm_vec_kernel<1024>, dim3(M), dim3(1024), 0, s, (bf16_t*)out, (const bf16_t*)z, z_ld, coef, eps, F);
+        else
+            hipLaunchKernelGGL(polynorm_vec_kernel<256>, dim3(M), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)z, z_ld, coef, eps, F);
+    } else if (dtype == PTA_BF16)
         hipLaunchKernelGGL(polynorm_kernel<bf16_t>, dim3(M), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)z, z_ld, coef, eps, F);
     else
         return pta_fail("polynorm: unknown dtype %d", dtype);

@@ -176,7 +176,7 @@ def test_scaled_embedding_with_learned_positions(dtype, rel):
 
 
 @pytest.mark.parametrize("dtype,rel", DTYPES)
-@pytest.mark.parametrize("ff,hidden", [(56, 40), (1, 8), (300, 24), (2048, 64)])
+@pytest.mark.parametrize("ff,hidden", [(56, 40), (1, 8), (300, 24), (2048, 64), (8200, 16), (12, 8)])
 def test_feed_forward_with_polynorm(dtype, rel, ff, hidden):
     from pytorch_transformers_amd.parts import PolyNormFeedForward
 
