@@ -1191,7 +1191,7 @@ def _talk_case(ops, nh, nkv, d, starts, news, cap=0.0, mix=True, window=0, chunk
         at += n
 
 
-TALK_SHAPES = [(8, 4, 48), (16, 8, 128), (4, 4, 64), (6, 2, 32), (3, 1, 16), (32, 8, 128), (16, 2, 64), (12, 12, 80),
+TALK_SHAPES = [(10, 5, 48), (16, 8, 128), (4, 4, 64), (6, 2, 32), (3, 1, 16), (32, 8, 128), (16, 2, 64), (12, 12, 80),
                (10, 2, 96), (2, 1, 112)]
 
 
@@ -1206,15 +1206,15 @@ def test_attn_talk_mfma_prompts_and_portions(nh, nkv, d):
     _talk_case(ops, nh, nkv, d, starts, news, cap=0.0, seed=1)
     _talk_case(ops, nh, nkv, d, starts, news, cap=0.0, mix=False, seed=2, loud=[3, 40, 100, 0, None, 70])
     _talk_case(ops, nh, nkv, d, starts, news, cap=2.0, mix=False, seed=3)
-    for window in (1, 33, 72):
+    for window in (1, 33, 70):
         _talk_case(ops, nh, nkv, d, starts, news, cap=4.0, window=window, seed=4)
     _talk_case(ops, nh, nkv, d, starts, news, cap=4.0, chunk=48, seed=5)
     for runs in (2, 3, 4):  # more runs than some tiles have blocks of keys
         _talk_case(ops, nh, nkv, d, starts, news, cap=5.0, seed=6, ranges=-runs)
-        _talk_case(ops, nh, nkv, d, starts, news, cap=5.0, window=72, seed=7, ranges=-runs)
+        _talk_case(ops, nh, nkv, d, starts, news, cap=5.0, window=70, seed=7, ranges=-runs)
 
 
-@pytest.mark.parametrize("nh,nkv,d", [(8, 4, 48), (16, 8, 128), (32, 8, 128), (16, 2, 64)])
+@pytest.mark.parametrize("nh,nkv,d", [(10, 5, 48), (16, 8, 128), (32, 8, 128), (16, 2, 64)])
 def test_attn_talk_mfma_long_prompts(nh, nkv, d):
     """A prompt of 700 tokens and 300 new tokens over 900 cached ones: many blocks of keys per workgroup, with and
     without a window."""
@@ -1247,7 +1247,7 @@ def test_attn_talk_mfma_sizes():
     assert not lib.pta_attn_talk_mfma_supported(34, 34, 64) and not lib.pta_attn_talk_mfma_supported(64, 8, 64)
     assert lib.pta_attn_talk_prompt_ranges(128, 2048) in (1, 2) and lib.pta_attn_talk_prompt_ranges(4096, 2048) == 1
     assert lib.pta_attn_talk_prompt_ranges(4, 100) == 1 and lib.pta_attn_talk_prompt_ranges(8, 5000) == 4
-    for n, length, window in ((1, 1, 0), (8, 1025, 1024), (64, 5000, 0), (3, 300000, 0), (512, 100, 72), (1, 70000, 1024)):
+    for n, length, window in ((1, 1, 0), (8, 1025, 1024), (64, 5000, 0), (3, 300000, 0), (512, 100, 70), (1, 70000, 1024)):
         ranges, size = ops.talk_decode_ranges(n, length, window)
         assert size % 64 == 0 and 1 <= ranges <= 1024 and ranges * size >= length
 
