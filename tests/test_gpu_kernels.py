@@ -1192,7 +1192,7 @@ def _talk_case(ops, nh, nkv, d, starts, news, cap=0.0, mix=True, window=0, chunk
 
 
 TALK_SHAPES = [(10, 5, 48), (16, 8, 128), (4, 4, 64), (6, 2, 32), (3, 1, 16), (32, 8, 128), (16, 2, 64), (12, 12, 80),
-               (10, 2, 96), (2, 1, 112)]
+               (10, 2, 96), (2, 1, 112), (24, 6, 96)]
 
 
 @pytest.mark.parametrize("nh,nkv,d", TALK_SHAPES)
