@@ -719,16 +719,20 @@ def attn_talk_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_
 
 
 def talk_decode_ranges(n_seqs: int, max_len: int, window: int = 0, chunk: int = 0) -> tuple:
-    """(ranges, keys a range) into which a decode step of ``attn_talk_mfma`` cuts the keys: about two workgroups for
-    every compute unit over the keys that a token sees at most, ranges of whole pages, at most 1,024 of them."""
+    """(runs, 0) for a decode step of ``attn_talk_mfma``: every token cuts the keys it sees into so many equal runs of
+    blocks, about two workgroups for every compute unit, a run no shorter than a page at the longest context, at most
+    1,024 runs and 65,535 workgroups a launch.  The size 0 says that the runs are each token's own (``attn_talk_mfma``):
+    what a window has left behind is in no run, so the partial results do not grow with the context.  The batch counts
+    by its next power of two and the longest context by its next multiple of 1,024, so that a captured step, which is
+    sized for a padded batch and such a bound, is cut exactly as the same step run directly."""
+    n_seqs = 1 << max(int(n_seqs) - 1, 0).bit_length()
+    max_len = (int(max_len) + 1023) // 1024 * 1024
     seen = max_len
     for bound in (window, chunk):
         if bound > 0:
-            seen = min(seen, bound + 63)
-    wanted = max(1, min((seen + 63) // 64, -(-512 // max(n_seqs, 1))))
-    size = (-(-seen // wanted) + 63) // 64 * 64
-    size = max(size, (-(-max_len // 1024) + 63) // 64 * 64)
-    return -(-max_len // size), size
+            seen = min(seen, bound + 31)
+    runs = min((seen + 63) // 64, -(-512 // max(n_seqs, 1)), 1024, 65535 // max(n_seqs, 1))
+    return max(1, runs), 0
 
 
 def attention_talk(q: torch.Tensor, k_pool, v_pool, block_table, ctx, scale: float, *, talk=None, softcap: float = 0.0,

@@ -1226,10 +1226,11 @@ def test_attn_talk_mfma_long_prompts(nh, nkv, d):
 
 
 @pytest.mark.parametrize("nh,nkv,d", TALK_SHAPES)
-@pytest.mark.parametrize("ranges", [None, 64, 256])
+@pytest.mark.parametrize("ranges", [None, 64, 256, -3, -17])
 def test_attn_talk_mfma_decode_ranges(nh, nkv, d, ranges):
-    """One token per sequence over contexts of very different lengths, the keys whole and cut into ranges that are
-    merged; ranges before a window and past a sequence's end; a loud far key."""
+    """One token per sequence over contexts of very different lengths, the keys whole, cut into ranges of the context
+    and into runs of each token's own keys (more of them than short contexts have blocks), merged; ranges before a
+    window and past a sequence's end; a loud far key."""
     ops = _ops()
     starts = [0, 63, 64, 700, 255, 256, 1, 1500]
     _talk_case(ops, nh, nkv, d, starts, [1] * 8, cap=5.0, ranges=ranges)
@@ -1247,9 +1248,15 @@ def test_attn_talk_mfma_sizes():
     assert not lib.pta_attn_talk_mfma_supported(34, 34, 64) and not lib.pta_attn_talk_mfma_supported(64, 8, 64)
     assert lib.pta_attn_talk_prompt_ranges(128, 2048) in (1, 2) and lib.pta_attn_talk_prompt_ranges(4096, 2048) == 1
     assert lib.pta_attn_talk_prompt_ranges(4, 100) == 1 and lib.pta_attn_talk_prompt_ranges(8, 5000) == 4
-    for n, length, window in ((1, 1, 0), (8, 1025, 1024), (64, 5000, 0), (3, 300000, 0), (512, 100, 70), (1, 70000, 1024)):
-        ranges, size = ops.talk_decode_ranges(n, length, window)
-        assert size % 64 == 0 and 1 <= ranges <= 1024 and ranges * size >= length
+    for n, length, window in ((1, 1, 0), (8, 1025, 1024), (64, 5000, 0), (3, 300000, 0), (512, 100, 70), (1, 70000, 1024),
+                              (4000, 90000, 0)):
+        runs, size = ops.talk_decode_ranges(n, length, window)
+        bound = (length + 1023) // 1024 * 1024
+        seen = min(bound, window + 31) if window else bound
+        assert size == 0 and 1 <= runs <= 1024 and runs * n <= max(65535, n) and runs <= (seen + 63) // 64
+        assert (runs, size) == ops.talk_decode_ranges(n, bound, window)  # a captured step's bound cuts the same way
+    assert ops.talk_decode_ranges(8, 1025, 1024)[0] == 17 and ops.talk_decode_ranges(1, 70000, 1024)[0] == 17
+    assert ops.talk_decode_ranges(5, 300, 0) == ops.talk_decode_ranges(8, 1024, 0)
 
 
 def test_decode_plan():
