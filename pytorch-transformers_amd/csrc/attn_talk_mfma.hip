@@ -2,6 +2,8 @@
 // attn_talk_mfma_impl.h, instantiated per head size in attn_talk_mfma_dt*.hip.
 #include "attn_talk_mfma_impl.h"
 
+#include <stdlib.h>
+
 #include <algorithm>
 
 #define PTA_TALK_HEAD(DT_) extern template bool talk_launch_head<DT_>(const TalkLaunch&, int);
@@ -14,7 +16,12 @@ static int talk_heads_per_wave(int nh, int nkv, int d) {
     if (nh <= 0 || nkv <= 0 || nh % nkv || d % 16 || d < 16 || d > 128) return 0;
     if ((size_t)nh * 4096 > 128 * 1024) return 0;  // the heads' tiles of two blocks of keys in LDS
     const int g = nh / nkv;
-    for (int ct = talk_max_heads(d / 16); ct >= 1; ct /= 2)
+    // PTA_TALK_HEADS: fewer heads a wave than the head size allows, for measurements (16 heads of 128 with a head a
+    // wave on sixteen waves: 156 us a layer of 2,048 tokens against 107 with two heads a wave on eight; every wave reads
+    // all heads' tiles, so twice the waves read twice as much from LDS)
+    static const int most_env = getenv("PTA_TALK_HEADS") ? atoi(getenv("PTA_TALK_HEADS")) : 0;
+    const int most = most_env > 0 ? std::min(most_env, talk_max_heads(d / 16)) : talk_max_heads(d / 16);
+    for (int ct = most; ct >= 1; ct /= 2)
         if (g % ct == 0 && nh / ct <= 16) return ct;
     return 0;
 }
