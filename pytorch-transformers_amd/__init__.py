@@ -6,6 +6,7 @@ from .engine import falcon as _falcon  # registers model_type "falcon"  # noqa: 
 from .engine import pavodra as _pavodra  # registers model_type "pavodra"  # noqa: F401
 from .engine import bimepel as _bimepel  # registers model_type "bimepel"  # noqa: F401
 from .engine import kekapel as _kekapel  # registers model_type "kekapel"  # noqa: F401
+from .engine import nopuzen as _nopuzen  # registers model_type "nopuzen"  # noqa: F401
 from .auto import AutoModelForCausalLM
 from .pipeline import TextGenerationPipeline, pipeline
 from .sampling.custom import LogitsProcessor, LogitsProcessorList, StoppingCriteria, StoppingCriteriaList

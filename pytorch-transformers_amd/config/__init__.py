@@ -4,8 +4,9 @@ from .falcon import FalconConfig
 from .pavodra import PavodraConfig
 from .bimepel import BimepelConfig
 from .kekapel import KekapelConfig
+from .nopuzen import NopuzenConfig
 from .generation import GENERATION_CONFIG_NAME, GenerationConfig
 from .registry import AutoConfig, known_model_types, lookup, register, unregister
 
-__all__ = ["CONFIG_NAME", "ConfigError", "ModelConfig", "FalconConfig", "PavodraConfig", "BimepelConfig", "KekapelConfig", "GENERATION_CONFIG_NAME", "GenerationConfig",
+__all__ = ["CONFIG_NAME", "ConfigError", "ModelConfig", "FalconConfig", "PavodraConfig", "BimepelConfig", "KekapelConfig", "NopuzenConfig", "GENERATION_CONFIG_NAME", "GenerationConfig",
            "AutoConfig", "known_model_types", "lookup", "register", "unregister"]

@@ -11,13 +11,13 @@
 #include "common.h"
 #include "pta_kernels.h"
 
-// One workgroup per token.  proj[t] = [q: H * (dn + dr) | down: R + dr] (row stride ld).
+// One workgroup per token.  q_rows[t] = H * (dn + dr) query elements (row stride q_ld), down_rows[t] = R + dr (row stride ld).
 //  - latent c = down[:R] / sqrt(mean(down[:R]^2) + eps) * w_norm -> cache row [0, R)
 //  - shared key part down[R:], its first rot->rotary_dim elements rotated by the token's position -> cache row [R, R + dr)
 //  - each head's rotated query part, rotated likewise -> q_full[t, h, R:]  (32-bit)
 template <typename T>
-__global__ void latent_prep_kernel(float* __restrict__ q_full, T* __restrict__ k_pool, const T* __restrict__ proj,
-                                   long ld, const float* __restrict__ w_norm, float eps,
+__global__ void latent_prep_kernel(float* __restrict__ q_full, T* __restrict__ k_pool, const T* __restrict__ q_rows,
+                                   long q_ld, const T* __restrict__ down_rows, long ld, const float* __restrict__ w_norm, float eps,
                                    const float* __restrict__ inv_freq, int inv_freq_ld, float cs_scale, int rot_n,
                                    int pairing, const int* __restrict__ token_pos, const int* __restrict__ token_seq,
                                    const int* __restrict__ block_table, int bt_stride, int H, int dn, int dr, int R,
@@ -25,8 +25,8 @@ __global__ void latent_prep_kernel(float* __restrict__ q_full, T* __restrict__ k
     __shared__ float red[16];
     const int m = blockIdx.x;
     const int pos = token_pos[m], seq = token_seq[m];
-    const T* row = proj + (long)m * ld;
-    const T* down = row + (long)H * (dn + dr);
+    const T* row = q_rows + (long)m * q_ld;
+    const T* down = down_rows + (long)m * ld;
     const float* freq = inv_freq ? inv_freq + (inv_freq_ld ? (long)seq * inv_freq_ld : 0) : nullptr;
     const int D = R + dr;
     // the element that element i of a rotated part is paired with, and the sign of the sine term
@@ -56,13 +56,16 @@ __global__ void latent_prep_kernel(float* __restrict__ q_full, T* __restrict__ k
     }
 }
 
-extern "C" int pta_latent_prep(float* q_full, void* k_pool, const void* proj, long ld, const float* w_norm, float eps,
+// q_rows [M, H * (dn + dr)] rows q_ld apart; down_rows [M, R + dr] rows ld apart (the two may be blocks of columns of
+// one product, or come from two)
+extern "C" int pta_latent_prep(float* q_full, void* k_pool, const void* q_rows, long q_ld, const void* proj, long ld,
+                               const float* w_norm, float eps,
                                const PtaRotation* rot, const int* token_pos, const int* token_seq,
                                const int* block_table, int bt_stride, int M, int H, int dn, int dr, int R,
                                int write_cache, int dtype, void* stream) {
     PTA_REQUIRE(M > 0 && H > 0 && dn > 0 && dr >= 0 && R > 0, "latent_prep: sizes must be positive");
-    PTA_REQUIRE(q_full && k_pool && proj && w_norm && token_pos && token_seq && block_table, "latent_prep: null pointer");
-    PTA_REQUIRE(ld >= (long)H * (dn + dr) + R + dr, "latent_prep: rows lie closer together than they are long");
+    PTA_REQUIRE(q_full && k_pool && q_rows && proj && w_norm && token_pos && token_seq && block_table, "latent_prep: null pointer");
+    PTA_REQUIRE(q_ld >= (long)H * (dn + dr) && ld >= (long)R + dr, "latent_prep: rows lie closer together than they are long");
     const float* inv_freq = rot ? rot->inv_freq : nullptr;
     int rot_n = 0, pairing = PTA_PAIR_HALF, freq_ld = 0;
     float cs = 1.f;
@@ -74,12 +77,12 @@ extern "C" int pta_latent_prep(float* q_full, void* k_pool, const void* proj, lo
     }
     hipStream_t s = (hipStream_t)stream;
     if (dtype == PTA_F32)
-        hipLaunchKernelGGL(latent_prep_kernel<float>, dim3(M), dim3(256), 0, s, q_full, (float*)k_pool, (const float*)proj,
-                           ld, w_norm, eps, inv_freq, freq_ld, cs, rot_n, pairing, token_pos, token_seq, block_table,
+        hipLaunchKernelGGL(latent_prep_kernel<float>, dim3(M), dim3(256), 0, s, q_full, (float*)k_pool, (const float*)q_rows,
+                           q_ld, (const float*)proj, ld, w_norm, eps, inv_freq, freq_ld, cs, rot_n, pairing, token_pos, token_seq, block_table,
                            bt_stride, H, dn, dr, R, write_cache);
     else if (dtype == PTA_BF16)
         hipLaunchKernelGGL(latent_prep_kernel<bf16_t>, dim3(M), dim3(256), 0, s, q_full, (bf16_t*)k_pool,
-                           (const bf16_t*)proj, ld, w_norm, eps, inv_freq, freq_ld, cs, rot_n, pairing, token_pos,
+                           (const bf16_t*)q_rows, q_ld, (const bf16_t*)proj, ld, w_norm, eps, inv_freq, freq_ld, cs, rot_n, pairing, token_pos,
                            token_seq, block_table, bt_stride, H, dn, dr, R, write_cache);
     else
         return pta_fail("latent_prep: unknown dtype %d", dtype);

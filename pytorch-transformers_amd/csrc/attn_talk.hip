@@ -4,6 +4,8 @@
 //   s_h <- softcap * tanh(s_h / softcap)              (softcap > 0)
 //   s_h <- sum over g of talk[h, g] * s_g             (talk given: [heads, heads], 32-bit)
 //   weights: softmax over the keys j that i sees (all before it, the last `window`, or its own block of `chunk`)
+//   (head_scale given: s_h is multiplied by head_scale[h] before the cap.  weights_kind PTA_WEIGHTS_SIGMOID: a key's
+//    weight is sigmoid(s_h + head_bias[h]), not normalised over the keys, in place of the softmax)
 //
 // The mix needs every head's score of a (query, key) pair in one place: a workgroup owns a token and all of its heads,
 // a wave a few heads.  Keys are taken a page (64) at a time from the first page the token sees, a lane a key; the
@@ -21,7 +23,9 @@ __global__ __launch_bounds__(1024) void attn_talk_kernel(T* __restrict__ out, co
                                                          const int* __restrict__ block_table, int bt_stride,
                                                          const int* __restrict__ token_seq, const int* __restrict__ token_pos,
                                                          const float* __restrict__ talk, float softcap, int nh, int nkv, int d,
-                                                         float scale, int window, int chunk) {
+                                                         float scale, int window, int chunk,
+                                                         const float* __restrict__ head_scale,
+                                                         const float* __restrict__ head_bias, int weights_kind) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
     float* q_s = sm;                    // [nh][d]
     float* raw_s = q_s + nh * d;        // [nh][64] capped scores of the page
@@ -63,6 +67,7 @@ __global__ __launch_bounds__(1024) void attn_talk_kernel(T* __restrict__ out, co
                     float dot = 0.f;
                     for (int i = 0; i < d; ++i) dot += qh[i] * Io<T>::ld(kr + i);
                     s = dot * scale;
+                    if (head_scale) s *= head_scale[h];
                     if (softcap > 0.f) s = softcap * tanhf(s * inv_cap);
                 }
                 raw_s[h * PTA_PAGE + lane] = s;
@@ -82,6 +87,10 @@ __global__ __launch_bounds__(1024) void attn_talk_kernel(T* __restrict__ out, co
                     for (int g = 0; g < nh; ++g) s += th[g] * raw_s[g * PTA_PAGE + lane];
                 } else {
                     s = raw_s[h * PTA_PAGE + lane];
+                }
+                if (weights_kind == PTA_WEIGHTS_SIGMOID) {
+                    p_s[h * PTA_PAGE + lane] = valid ? 1.0f / (1.0f + expf(-(s + (head_bias ? head_bias[h] : 0.f)))) : 0.f;
+                    continue;
                 }
                 if (!valid) s = -INFINITY;
                 const float m_new = fmaxf(m_run[r], wave_max(s));
@@ -118,7 +127,7 @@ __global__ __launch_bounds__(1024) void attn_talk_kernel(T* __restrict__ out, co
         const int h = wave + r * nw;
         if (h < nh) {
             T* orow = out + ((long)m * nh + h) * d;
-            const float inv = 1.0f / l_run[r];
+            const float inv = weights_kind == PTA_WEIGHTS_SIGMOID ? 1.0f : 1.0f / l_run[r];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const int dim = lane + c * PTA_WAVE;
@@ -140,7 +149,9 @@ extern "C" int pta_attn_talk_sizes_ok(int nh, int nkv, int d) {
 
 extern "C" int pta_attn_talk(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                              int bt_stride, const int* token_seq, const int* token_pos, const float* talk, float softcap, int M,
-                             int nh, int nkv, int d, float scale, int window, int chunk, int dtype, void* stream) {
+                             int nh, int nkv, int d, float scale, int window, int chunk, const float* head_scale,
+                             const float* head_bias, int weights_kind, int dtype, void* stream) {
+    PTA_REQUIRE(weights_kind == PTA_WEIGHTS_SOFTMAX || weights_kind == PTA_WEIGHTS_SIGMOID, "attn_talk: weights of kind %d are not built", weights_kind);
     PTA_REQUIRE(M > 0, "attn_talk: no tokens");
     if (pta_attn_talk_sizes_ok(nh, nkv, d)) return 1;
     PTA_REQUIRE(window >= 0 && chunk >= 0 && softcap >= 0.f, "attn_talk: window, chunk and softcap are 0 (none) or positive");
@@ -151,7 +162,7 @@ extern "C" int pta_attn_talk(void* out, const void* q, const void* k_pool, const
 #define PTA_TALK(T, R)                                                                                                    \
     hipLaunchKernelGGL((attn_talk_kernel<T, R>), dim3(M), dim3(waves * PTA_WAVE), lds, s, (T*)out, (const T*)q,            \
                        (const T*)k_pool, (const T*)v_pool, block_table, bt_stride, token_seq, token_pos, talk, softcap, nh, \
-                       nkv, d, scale, window, chunk)
+                       nkv, d, scale, window, chunk, head_scale, head_bias, weights_kind)
 #define PTA_TALK_R(T)                       \
     do {                                    \
         if (hpw == 1) PTA_TALK(T, 1);       \

@@ -39,7 +39,9 @@ extern "C" int pta_attn_talk_mfma_supported(int nh, int nkv, int d) { return tal
 extern "C" int pta_attn_talk_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                                   int bt_stride, const int* cu_tokens, const int* seq_start, const float* talk, float softcap,
                                   int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int window, int chunk,
-                                  int split_size, int n_splits, float* po, float* pm, float* pl, void* stream) {
+                                  int split_size, int n_splits, float* po, float* pm, float* pl, const float* head_scale,
+                                  const float* head_bias, int weights_kind, void* stream) {
+    PTA_REQUIRE(weights_kind == PTA_WEIGHTS_SOFTMAX || weights_kind == PTA_WEIGHTS_SIGMOID, "attn_talk_mfma: weights of kind %d are not built", weights_kind);
     PTA_REQUIRE(n_seqs > 0 && max_new > 0 && M > 0, "attn_talk_mfma: sizes must be positive");
     const int ct = talk_heads_per_wave(nh, nkv, d);
     PTA_REQUIRE(ct > 0, "attn_talk_mfma: %d heads on %d KV heads of size %d are not built (sizes 16..128 in steps of 16, "
@@ -57,7 +59,7 @@ extern "C" int pta_attn_talk_mfma(void* out, const void* q, const void* k_pool, 
     const float pre_mul = softcap > 0.f ? 2.0f * scale * TALK_LOG2E / softcap : scale;
     const TalkLaunch a{(bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table,
                        bt_stride, cu_tokens, seq_start, talk, softcap, pre_mul, n_seqs, max_new, nh, nkv, window, chunk,
-                       split_size, n_splits, (hipStream_t)stream};
+                       split_size, n_splits, (hipStream_t)stream, head_scale, head_bias, weights_kind};
     bool built = false;
     switch (d / 16) {
 #define PTA_TALK_CASE(DT_) case DT_: built = talk_launch_head<DT_>(a, ct); break;

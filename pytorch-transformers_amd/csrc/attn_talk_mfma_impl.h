@@ -2,6 +2,8 @@
 // (the arithmetic of attn_talk.hip), bfloat16 in, on the matrix cores; prompts and decode steps are the same code.
 //
 //   s_h(i, j) = q_h(i) . k(j) * scale;  s_h <- cap * tanh(s_h / cap);  s_h <- sum over g of talk[h, g] * s_g
+//   (head_scale given: s_h is multiplied by head_scale[h] before the cap.  weights_kind PTA_WEIGHTS_SIGMOID: a key's
+//    weight is sigmoid(s_h + head_bias[h]), not normalised over the keys, in place of the softmax)
 //
 // The mix needs every head's score of a (query, key) pair in one place.  A workgroup owns sixteen consecutive tokens
 // of one sequence and all heads; a wave owns CT heads of one KV head.  Keys are walked 32 at a time:
@@ -55,7 +57,8 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool,
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ cu_tokens,
     const int* __restrict__ seq_start, const float* __restrict__ talk, float cap, float pre_mul, int nh, int nkv,
-    int window, int chunk, int split_size, int n_splits) {
+    int window, int chunk, int split_size, int n_splits, const float* __restrict__ head_scale,
+    const float* __restrict__ head_bias, int weights_kind) {
     constexpr int D = DT * 16, DS = (DT + 1) / 2, CHUNKS = D / 8;
     extern __shared__ __attribute__((aligned(16))) float4 talk_tiles[];  // [2][nh][2][64], then the mix [nh][nh]
     auto lowest_key = [&](int t) {
@@ -114,9 +117,12 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
         }
     }
     talk_f32x4_t oacc[DT][CT], lacc[CT];
-    float m_run[CT], m_raise[CT];
+    float m_run[CT], m_raise[CT], mul_h[CT], bias_h[CT];
+    const bool sig = weights_kind == PTA_WEIGHTS_SIGMOID;
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
+        mul_h[ct] = head_scale ? pre_mul * head_scale[h0 + ct] : pre_mul;
+        bias_h[ct] = head_bias ? head_bias[h0 + ct] * TALK_LOG2E : 0.f;
         m_run[ct] = -INFINITY;
         m_raise[ct] = -INFINITY;
         lacc[ct] = talk_f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -180,7 +186,7 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
             for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float x = s[tt][ct][e] * pre_mul;
+                    float x = s[tt][ct][e] * mul_h[ct];
                     // cap * tanh(z) = cap - 2 cap / (1 + e^(2z)); pre_mul carries 2 scale log2(e) / cap
                     if (cap > 0.f) x = __builtin_fmaf(cap2, __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x)), cap);
                     s[tt][ct][e] = x;
@@ -238,6 +244,15 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
                 for (int j = 0; j < 8; ++j)
                     if (kb + 8 * gq + j >= lim || kb + 8 * gq + j < lo) s[j >> 2][ct][j & 3] = -INFINITY;
             }
+            if (sig) {  // 1 / (1 + 2^(-(s + bias) log2 e)); a key that is not seen has s = -inf and the weight 0
+                float p[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    p[j] = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-__builtin_fmaf(s[j >> 2][ct][j & 3], TALK_LOG2E, bias_h[ct])));
+                pf[ct].u = make_uint4(talk_pack_bf16(p[0], p[1]), talk_pack_bf16(p[2], p[3]), talk_pack_bf16(p[4], p[5]),
+                                      talk_pack_bf16(p[6], p[7]));
+                continue;
+            }
             float mx = fmaxf(fmaxf(fmaxf(s[0][ct][0], s[0][ct][1]), fmaxf(s[0][ct][2], s[0][ct][3])),
                              fmaxf(fmaxf(s[1][ct][0], s[1][ct][1]), fmaxf(s[1][ct][2], s[1][ct][3])));
             // The running maximum is a reference point for the exponentials, shared by the four lanes of a column;
@@ -263,9 +278,11 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
             pf[ct].u = make_uint4(talk_pack_bf16(p[0], p[1]), talk_pack_bf16(p[2], p[3]), talk_pack_bf16(p[4], p[5]),
                                   talk_pack_bf16(p[6], p[7]));
         }
+        if (!sig) {
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
-            lacc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pf[ct].v, lacc[ct], 0, 0, 0);
+            for (int ct = 0; ct < CT; ++ct)
+                lacc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones.v, pf[ct].v, lacc[ct], 0, 0, 0);
+        }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -276,7 +293,9 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         if (qpos < 0) continue;
-        const float l = lacc[ct][0];
+        // (unnormalised weights: the ranges' sums are added as they are, which the merge does when every range that has
+        // keys says maximum 0 and exactly one of them, the one that holds the token's own position, weight sum 1)
+        const float l = sig ? ((n_splits == 1 || (qpos >= k_begin && qpos < k_end)) ? 1.f : 0.f) : lacc[ct][0];
         const long row = (long)tok * nh + h0 + ct;
         if (n_splits == 1) {
             const float inv = 1.0f / l;
@@ -295,7 +314,7 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
                 *reinterpret_cast<float4*>(o + dt * 16 + gq * 4) =
                     make_float4(oacc[dt][ct][0], oacc[dt][ct][1], oacc[dt][ct][2], oacc[dt][ct][3]);
             if (gq == 0) {
-                pm[row * n_splits + split] = m_run[ct];
+                pm[row * n_splits + split] = sig ? 0.f : m_run[ct];
                 pl[row * n_splits + split] = l;
             }
         }
@@ -309,6 +328,7 @@ struct TalkLaunch {
     const int *cu_tokens, *seq_start; const float* talk; float cap, pre_mul;
     int n_seqs, max_new, nh, nkv, window, chunk, split_size, n_splits;
     hipStream_t s;
+    const float *head_scale, *head_bias; int weights_kind;
 };
 
 // heads that one wave may hold at this head size (the registers of the sums set it)
@@ -330,7 +350,7 @@ static void talk_launch_one(const TalkLaunch& a) {
     const dim3 grid((a.max_new + 15) / 16, a.n_seqs * a.n_splits);
     hipLaunchKernelGGL(kern, grid, dim3(64 * (a.nh / CT)), lds, a.s, a.out, a.po, a.pm, a.pl, a.q, a.k_pool, a.v_pool,
                        a.block_table, a.bt_stride, a.cu_tokens, a.seq_start, a.talk, a.cap, a.pre_mul, a.nh, a.nkv, a.window,
-                       a.chunk, a.split_size, a.n_splits);
+                       a.chunk, a.split_size, a.n_splits, a.head_scale, a.head_bias, a.weights_kind);
 }
 
 // What pta_attn_talk_mfma launches for heads of DT x 16 elements with `ct` heads a wave; every head size is a

@@ -152,6 +152,11 @@ __device__ __forceinline__ float apply_act(float x, int act) {
     }
 }
 
+// xIELU with its two coefficients already formed: z > 0: ap z^2 + z / 2; z <= 0: an (e^z - 1 - z) + z / 2
+__device__ __forceinline__ float xielu_value(float z, float ap, float an) {
+    return z > 0.f ? __builtin_fmaf(ap * z, z, 0.5f * z) : __builtin_fmaf(an, expm1f(z) - z, 0.5f * z);
+}
+
 // act(g) * u, or the clamped gate (kinds and fields: PtaGate in pta_kernels.h), in 32-bit
 template <typename Gate>
 __device__ __forceinline__ float gate_value(float g, float u, int act, const Gate& how) {

@@ -2,7 +2,10 @@
 //
 // pta_gated_heads:  out[m, h * dv + e] = n(x)[m, h, e] * sigmoid(g[m, h * dv + e]), where x holds heads of dv elements
 //                   in frames x_head apart (an attention result whose frames are wider than its values), and n is
-//                   the identity or an RMS norm over the whole row of heads * dv elements with a weight.
+//                   the identity or an RMS norm over the whole row of heads * dv elements with a weight.  With
+//                   g_per_head the gate is one number a head: sigmoid(g[m, h]).
+// pta_xielu:        out[m, f] = z > 0 ? ap * z^2 + z / 2 : an * (e^z - 1 - z) + z / 2 with ap = softplus(act[0]) and
+//                   an = 1/2 + softplus(act[1]), act two learned numbers held in 32-bit.
 // pta_glu:          out[m, f] = act(gate[m, f], up[m, f]) for a feed-forward with a gate:
 //                   PTA_GLU_SILU        silu(gate) * up
 //                   PTA_GLU_CLAMPED     g = min(gate, limit), u = clamp(up, -limit, limit): g * sigmoid(alpha g) * (u + 1)
@@ -15,7 +18,8 @@
 template <typename T, typename TX>
 __global__ __launch_bounds__(1024) void gated_heads_kernel(T* __restrict__ out, const TX* __restrict__ x, long x_ld,
                                                           int x_head, const T* __restrict__ g, long g_ld,
-                                                          const float* __restrict__ w, float eps, int heads, int dv) {
+                                                          const float* __restrict__ w, float eps, int heads, int dv,
+                                                          int g_per_head) {
     __shared__ float red[16];
     const int m = blockIdx.x, N = heads * dv;
     const TX* xr = x + (long)m * x_ld;
@@ -31,30 +35,30 @@ __global__ __launch_bounds__(1024) void gated_heads_kernel(T* __restrict__ out, 
     for (int i = threadIdx.x; i < N; i += blockDim.x) {
         float v = Io<TX>::ld(xr + (long)(i / dv) * x_head + i % dv);
         if (w) v = v * inv * w[i];
-        const float gate = 1.0f / (1.0f + expf(-Io<T>::ld(g + (long)m * g_ld + i)));
+        const float gate = 1.0f / (1.0f + expf(-Io<T>::ld(g + (long)m * g_ld + (g_per_head ? i / dv : i))));
         Io<T>::st(out + (long)m * N + i, v * gate);
     }
 }
 
 // x: 32-bit (x_f32) or the compute type; g and out in the compute type
 extern "C" int pta_gated_heads(void* out, const void* x, int x_f32, long x_ld, int x_head, const void* g, long g_ld,
-                               const float* w, float eps, int M, int heads, int dv, int dtype, void* stream) {
+                               const float* w, float eps, int M, int heads, int dv, int g_per_head, int dtype, void* stream) {
     PTA_REQUIRE(M > 0 && heads > 0 && dv > 0, "gated_heads: sizes must be positive");
     PTA_REQUIRE(out && x && g, "gated_heads: null pointer");
-    PTA_REQUIRE(x_head >= dv && x_ld >= (long)(heads - 1) * x_head + dv && g_ld >= (long)heads * dv,
+    PTA_REQUIRE(x_head >= dv && x_ld >= (long)(heads - 1) * x_head + dv && g_ld >= (long)heads * (g_per_head ? 1 : dv),
                 "gated_heads: rows or frames lie closer together than they are long");
     PTA_REQUIRE(dtype == PTA_F32 || dtype == PTA_BF16, "gated_heads: unknown dtype %d", dtype);
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid(M), block(std::min(1024, std::max(64, (heads * dv / 4 + 63) / 64 * 64)));
     if (dtype == PTA_F32)
         hipLaunchKernelGGL((gated_heads_kernel<float, float>), grid, block, 0, s, (float*)out, (const float*)x, x_ld, x_head,
-                           (const float*)g, g_ld, w, eps, heads, dv);
+                           (const float*)g, g_ld, w, eps, heads, dv, g_per_head);
     else if (x_f32)
         hipLaunchKernelGGL((gated_heads_kernel<bf16_t, float>), grid, block, 0, s, (bf16_t*)out, (const float*)x, x_ld, x_head,
-                           (const bf16_t*)g, g_ld, w, eps, heads, dv);
+                           (const bf16_t*)g, g_ld, w, eps, heads, dv, g_per_head);
     else
         hipLaunchKernelGGL((gated_heads_kernel<bf16_t, bf16_t>), grid, block, 0, s, (bf16_t*)out, (const bf16_t*)x, x_ld,
-                           x_head, (const bf16_t*)g, g_ld, w, eps, heads, dv);
+                           x_head, (const bf16_t*)g, g_ld, w, eps, heads, dv, g_per_head);
     return pta_check_launch("gated_heads");
 }
 
@@ -90,6 +94,31 @@ extern "C" int pta_glu(void* out, const void* gate, const void* up, long in_ld, 
     else
         hipLaunchKernelGGL(glu_kernel<bf16_t>, grid, dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)gate, (const bf16_t*)up, in_ld, F, n, kind, alpha, limit);
     return pta_check_launch("glu");
+}
+
+// z: [M, F] with rows z_ld apart; out [M, F] dense.  softplus in 32-bit (the identity beyond 20, where 1 + e^v rounds to e^v).
+__device__ __forceinline__ float softplus_f32(float v) { return v > 20.f ? v : log1pf(expf(v)); }
+
+template <typename T>
+__global__ void xielu_kernel(T* __restrict__ out, const T* __restrict__ z, long z_ld, int F, long n,
+                             const float* __restrict__ act) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const long m = i / F, f = i - m * F;
+    Io<T>::st(out + i, xielu_value(Io<T>::ld(z + m * z_ld + f), softplus_f32(act[0]), 0.5f + softplus_f32(act[1])));
+}
+
+extern "C" int pta_xielu(void* out, const void* z, long z_ld, int M, int F, const float* act, int dtype, void* stream) {
+    PTA_REQUIRE(M > 0 && F > 0 && out && z && act && z_ld >= F, "xielu: sizes must be positive and pointers given");
+    PTA_REQUIRE(dtype == PTA_F32 || dtype == PTA_BF16, "xielu: unknown dtype %d", dtype);
+    hipStream_t s = (hipStream_t)stream;
+    const long n = (long)M * F;
+    const dim3 grid((unsigned)((n + 255) / 256));
+    if (dtype == PTA_F32)
+        hipLaunchKernelGGL(xielu_kernel<float>, grid, dim3(256), 0, s, (float*)out, (const float*)z, z_ld, F, n, act);
+    else
+        hipLaunchKernelGGL(xielu_kernel<bf16_t>, grid, dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)z, z_ld, F, n, act);
+    return pta_check_launch("xielu");
 }
 
 // PolyNorm (see pta_kernels.h): one workgroup per row, the three mean squares in one pass, the row read again for the

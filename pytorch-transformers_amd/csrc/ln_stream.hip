@@ -7,7 +7,7 @@
 //   s += add                               another 32-bit tensor of the stream's shape (rows of its own), if given
 //   s += vec                               one 32-bit vector for every row, if given
 //   out_wide = s                           if wanted
-//   out_narrow = LN(s) * w + b             in the compute type, if w is given
+//   out_narrow = LN(s) * w + b             in the compute type, if w is given; without w, s itself in the compute type
 //
 // `rows` gathers: output row m is made of input row rows[m] (the final norm on the wanted rows alone).
 // One workgroup per row; a thread keeps its VPT elements in registers over all passes; every sum over a row is taken
@@ -78,7 +78,16 @@ __global__ __launch_bounds__(256) void layernorm_stream_kernel(T* __restrict__ o
             if (i < H) out_wide[(long)m * H + i] = s[k];
         }
     }
-    if (!w) return;
+    if (!w) {
+        if (out_narrow) {
+#pragma unroll
+            for (int k = 0; k < VPT; ++k) {
+                const int i = threadIdx.x + k * blockDim.x;
+                if (i < H) Io<T>::st(out_narrow + (long)m * H + i, s[k]);
+            }
+        }
+        return;
+    }
     float wv[VPT], bv[VPT];
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
@@ -137,7 +146,7 @@ extern "C" int pta_layernorm_stream(void* out_narrow, float* out_wide, const flo
     PTA_REQUIRE(x || y, "layernorm_stream: neither a stream nor a sublayer's output given");
     PTA_REQUIRE(!y || (wy && by && y_ld >= H), "layernorm_stream: a sublayer's output needs its norm's weight and bias");
     PTA_REQUIRE((w != nullptr) == (b != nullptr), "layernorm_stream: weight and bias come together");
-    PTA_REQUIRE((w != nullptr) == (out_narrow != nullptr), "layernorm_stream: the normed output and its weight come together");
+    PTA_REQUIRE(!w || out_narrow, "layernorm_stream: a norm of the stream needs a place for its output");
     PTA_REQUIRE(out_narrow || out_wide, "layernorm_stream: nothing to write");
     hipStream_t s = (hipStream_t)stream;
     if (dtype == PTA_F32)

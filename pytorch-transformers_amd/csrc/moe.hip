@@ -3,7 +3,11 @@
 //   z = W_r h (32-bit); s = score(z) (sigmoid, or softmax over the experts); the `top` largest s are taken;
 //   weights = s / (sum of the taken s + 1e-20) * scale   (or the taken s times scale, unnormalised);
 //   out = sum over the taken experts e of weight_e * D_e (act(G_e h) * (U_e h))
-//   (z may have a bias added; in place of act(g) * u an expert may have the clamped gate of PtaGate, pta_kernels.h)
+//   (z may have a bias added; in place of act(g) * u an expert may have the clamped gate of PtaGate, pta_kernels.h;
+//    an expert without a gate is D_e act(U_e h), its matrices stacked as up [E, F, H]; with groups the experts form
+//    `groups` equal runs of neighbours, a run's score is its largest s, and only experts of the `keep` best runs can
+//    be taken; the router's launch can also form sigmoid(X h) for a few more 32-bit rows X, e.g. the gate of an expert
+//    that every token uses, whose output the launch that sums the taken experts adds times that gate)
 //
 // Expert matrices are held stacked: gate_up [E, 2F, H] (an expert's gate rows, then its up rows) and down [E, H, F].
 //
@@ -80,7 +84,9 @@ template <typename T>
 __global__ __launch_bounds__(1024) void moe_route_kernel(int* __restrict__ ids, float* __restrict__ wts,
                                                         const T* __restrict__ h, long h_ld, const float* __restrict__ Wr,
                                                         const float* __restrict__ br, int H, int E, int top, int score_kind,
-                                                        int normalise, float scale) {
+                                                        int normalise, float scale, int groups, int keep,
+                                                        const float* __restrict__ extra, float* __restrict__ extra_out,
+                                                        int n_extra) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
     float* x_s = sm;       // [H]
     float* s_s = sm + H;   // [E]
@@ -90,6 +96,10 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(int* __restrict__ ids, 
     for (int e = wave; e < E; e += nw) {
         const float z = wave_dot<float>(Wr + (long)e * H, x_s, H, lane);
         if (lane == 0) s_s[e] = br ? z + br[e] : z;
+    }
+    for (int e = wave; e < n_extra; e += nw) {
+        const float z = wave_dot<float>(extra + (long)e * H, x_s, H, lane);
+        if (lane == 0) extra_out[(long)m * n_extra + e] = 1.0f / (1.0f + expf(-z));
     }
     __syncthreads();
     if (wave != 0) return;
@@ -107,7 +117,29 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(int* __restrict__ ids, 
     // the largest score `top` times over; of equal scores the expert with the lower index first
     float total = 0.f, mine = 0.f;
     int mine_id = 0;
-    unsigned taken = 0;  // bit j: this lane's expert lane + 64 j has been taken
+    unsigned taken = 0;  // bit j: this lane's expert lane + 64 j has been taken (or may not be)
+    if (groups > 1 && keep < groups) {
+        // lane g holds the score of run g (at most 64 runs); the `keep` best runs stay, the lower index first among equals
+        const int size = E / groups;
+        float gs = -INFINITY;
+        if (lane < groups)
+            for (int e = lane * size; e < (lane + 1) * size; ++e) gs = fmaxf(gs, s_s[e]);
+        unsigned long long kept = 0ull;
+        for (int k = 0; k < keep; ++k) {
+            float best = gs;
+            int at = lane < groups && !((kept >> lane) & 1ull) ? lane : groups;
+            if (at == groups) best = -INFINITY;
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ob = __shfl_xor(best, o, 64);
+                const int oa = __shfl_xor(at, o, 64);
+                if (oa < groups && (at == groups || ob > best || (ob == best && oa < at))) { best = ob; at = oa; }
+            }
+            kept |= 1ull << at;
+        }
+        for (int e = lane, j = 0; e < E; e += PTA_WAVE, ++j)
+            if (!((kept >> (e / size)) & 1ull)) taken |= 1u << j;
+    }
     for (int k = 0; k < top; ++k) {
         float best = -INFINITY;
         int at = E;
@@ -132,10 +164,14 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(int* __restrict__ ids, 
 }
 
 extern "C" int pta_moe_route(int* ids, float* wts, const void* h, long h_ld, const float* Wr, const float* br, int M, int H, int E, int top,
-                             int score_kind, int normalise, float scale, int dtype, void* stream) {
+                             int score_kind, int normalise, float scale, int groups, int keep, const float* extra,
+                             float* extra_out, int n_extra, int dtype, void* stream) {
     PTA_REQUIRE(M > 0 && H > 0 && E > 0 && top > 0, "moe_route: sizes must be positive");
     PTA_REQUIRE(top <= E && top <= 64 && E <= 2048, "moe_route: %d experts per token of %d (at most 64 of at most 2048)", top, E);
     PTA_REQUIRE(ids && wts && h && Wr && h_ld >= H, "moe_route: null pointer or rows too close");
+    PTA_REQUIRE(groups >= 1 && groups <= 64 && E % groups == 0 && keep >= 1 && keep <= groups && (long)keep * (E / groups) >= top,
+                "moe_route: %d experts in %d groups of which %d are kept do not give %d experts a token", E, groups, keep, top);
+    PTA_REQUIRE(n_extra >= 0 && (n_extra == 0 || (extra && extra_out)), "moe_route: further rows need their matrix and a place for the result");
     PTA_REQUIRE(score_kind == PTA_ROUTE_SIGMOID || score_kind == PTA_ROUTE_SOFTMAX, "moe_route: score kind %d is not built", score_kind);
     PTA_REQUIRE((size_t)(H + E) * 4 <= 64 * 1024, "moe_route: %d features and %d experts do not fit the kernel's LDS", H, E);
     PTA_REQUIRE(dtype == PTA_F32 || dtype == PTA_BF16, "moe_route: unknown dtype %d", dtype);
@@ -143,9 +179,9 @@ extern "C" int pta_moe_route(int* ids, float* wts, const void* h, long h_ld, con
     const size_t lds = (size_t)(H + E) * sizeof(float);
     const dim3 block(E >= 16 ? 1024 : E >= 8 ? 512 : 256);  // a wave an expert where there are that many
     if (dtype == PTA_F32)
-        hipLaunchKernelGGL(moe_route_kernel<float>, dim3(M), block, lds, s, ids, wts, (const float*)h, h_ld, Wr, br, H, E, top, score_kind, normalise, scale);
+        hipLaunchKernelGGL(moe_route_kernel<float>, dim3(M), block, lds, s, ids, wts, (const float*)h, h_ld, Wr, br, H, E, top, score_kind, normalise, scale, groups, keep, extra, extra_out, n_extra);
     else
-        hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(M), block, lds, s, ids, wts, (const bf16_t*)h, h_ld, Wr, br, H, E, top, score_kind, normalise, scale);
+        hipLaunchKernelGGL(moe_route_kernel<bf16_t>, dim3(M), block, lds, s, ids, wts, (const bf16_t*)h, h_ld, Wr, br, H, E, top, score_kind, normalise, scale, groups, keep, extra, extra_out, n_extra);
     return pta_check_launch("moe_route");
 }
 
@@ -154,19 +190,29 @@ extern "C" int pta_moe_route(int* ids, float* wts, const void* h, long h_ld, con
 template <typename T>
 __global__ __launch_bounds__(256) void moe_up_kernel(T* __restrict__ act_out, const T* __restrict__ h, long h_ld,
                                                      const T* __restrict__ gate_up, const int* __restrict__ ids, int H,
-                                                     int F, int top, int act, PtaGate gate) {
+                                                     int F, int top, int act, PtaGate gate, int gated) {
     extern __shared__ __attribute__((aligned(16))) float x_s[];  // [H]
     const int pair = blockIdx.x, m = pair / top, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int e = ids[pair];
     for (int i = threadIdx.x; i < H; i += blockDim.x) x_s[i] = Io<T>::ld(h + (long)m * h_ld + i);
     __syncthreads();
-    const T* G = gate_up + (long)e * 2 * F * H;
+    const T* G = gate_up + (long)e * (gated ? 2 : 1) * F * H;
     const T* U = G + (long)F * H;
     // a wave takes four neighbouring rows of the gate and of the up matrix: eight loads on their way at once
     const int f0 = blockIdx.y * MOE_ROWS + wave * 4, rows = min(4, F - f0);
     if (rows <= 0) return;
     float g[4], u[4];
     wave_dots<T, 4>(G + (long)f0 * H, H, rows, x_s, H, lane, g);
+    if (!gated) {  // an expert without a gate: act of its one product
+        if (lane < rows) {
+            float gv = g[0];
+#pragma unroll
+            for (int r = 1; r < 4; ++r)
+                if (lane == r) gv = g[r];
+            Io<T>::st(act_out + (long)pair * F + f0 + lane, apply_act(Io<T>::round(gv), act));
+        }
+        return;
+    }
     wave_dots<T, 4>(U + (long)f0 * H, H, rows, x_s, H, lane, u);
     // (each product rounded to the compute type first, as a product on its own would leave it)
     if (lane < rows) {
@@ -181,7 +227,9 @@ __global__ __launch_bounds__(256) void moe_up_kernel(T* __restrict__ act_out, co
 template <typename T>
 __global__ __launch_bounds__(256) void moe_down_kernel(T* __restrict__ out, const T* __restrict__ act_in,
                                                        const T* __restrict__ down, const int* __restrict__ ids,
-                                                       const float* __restrict__ wts, int H, int F, int top) {
+                                                       const float* __restrict__ wts, int H, int F, int top,
+                                                       const T* __restrict__ extra, const float* __restrict__ extra_gate,
+                                                       int gate_ld) {
     extern __shared__ __attribute__((aligned(16))) float a_s[];  // [top][F]
     const int m = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int i = threadIdx.x; i < top * F; i += blockDim.x) a_s[i] = Io<T>::ld(act_in + (long)m * top * F + i);
@@ -201,13 +249,14 @@ __global__ __launch_bounds__(256) void moe_down_kernel(T* __restrict__ out, cons
 #pragma unroll
         for (int r = 1; r < 4; ++r)
             if (lane == r) v = acc[r];
+        if (extra) v += extra_gate[(long)m * gate_ld] * Io<T>::ld(extra + (long)m * H + n0 + lane);
         Io<T>::st(out + (long)m * H + n0 + lane, v);
     }
 }
 
-// act_out [M * top, F]; h [M, H] rows h_ld apart; gate_up [E, 2F, H]; ids [M, top]
+// act_out [M * top, F]; h [M, H] rows h_ld apart; gate_up [E, 2F, H] (gated) or [E, F, H]; ids [M, top]
 extern "C" int pta_moe_up(void* act_out, const void* h, long h_ld, const void* gate_up, const int* ids, int M, int H, int F,
-                          int top, int act, const PtaGate* gate_how, int dtype, void* stream) {
+                          int top, int act, const PtaGate* gate_how, int gated, int dtype, void* stream) {
     const PtaGate gate = gate_how ? *gate_how : PtaGate{PTA_GLU_SILU, 1.f, 0.f};
     PTA_REQUIRE(gate.kind == PTA_GLU_SILU || gate.kind == PTA_GLU_CLAMPED, "moe_up: a gate of kind %d is not built", gate.kind);
     PTA_REQUIRE(M > 0 && H > 0 && F > 0 && top > 0 && act_out && h && gate_up && ids && h_ld >= H, "moe_up: sizes must be positive and pointers given");
@@ -217,15 +266,17 @@ extern "C" int pta_moe_up(void* act_out, const void* h, long h_ld, const void* g
     hipStream_t s = (hipStream_t)stream;
     const dim3 grid((unsigned)((long)M * top), (F + MOE_ROWS - 1) / MOE_ROWS);
     if (dtype == PTA_F32)
-        hipLaunchKernelGGL(moe_up_kernel<float>, grid, dim3(256), (size_t)H * 4, s, (float*)act_out, (const float*)h, h_ld, (const float*)gate_up, ids, H, F, top, act, gate);
+        hipLaunchKernelGGL(moe_up_kernel<float>, grid, dim3(256), (size_t)H * 4, s, (float*)act_out, (const float*)h, h_ld, (const float*)gate_up, ids, H, F, top, act, gate, gated);
     else
-        hipLaunchKernelGGL(moe_up_kernel<bf16_t>, grid, dim3(256), (size_t)H * 4, s, (bf16_t*)act_out, (const bf16_t*)h, h_ld, (const bf16_t*)gate_up, ids, H, F, top, act, gate);
+        hipLaunchKernelGGL(moe_up_kernel<bf16_t>, grid, dim3(256), (size_t)H * 4, s, (bf16_t*)act_out, (const bf16_t*)h, h_ld, (const bf16_t*)gate_up, ids, H, F, top, act, gate, gated);
     return pta_check_launch("moe_up");
 }
 
 // out [M, H]; act_in [M * top, F]; down [E, H, F]
+// extra [M, H] (compute type) and extra_gate (32-bit, one number a token, gate_ld apart), both or neither: out += gate * extra
 extern "C" int pta_moe_down(void* out, const void* act_in, const void* down, const int* ids, const float* wts, int M, int H,
-                            int F, int top, int dtype, void* stream) {
+                            int F, int top, const void* extra, const float* extra_gate, int gate_ld, int dtype, void* stream) {
+    PTA_REQUIRE((extra != nullptr) == (extra_gate != nullptr), "moe_down: a further term and its gate come together");
     PTA_REQUIRE(M > 0 && H > 0 && F > 0 && top > 0 && out && act_in && down && ids && wts, "moe_down: sizes must be positive and pointers given");
     PTA_REQUIRE((size_t)top * F * 4 <= 160 * 1024 && (H + MOE_ROWS - 1) / MOE_ROWS <= 65535,
                 "moe_down: %d experts of %d rows a token are more than the kernel's LDS holds", top, F);
@@ -238,9 +289,9 @@ extern "C" int pta_moe_down(void* out, const void* act_in, const void* down, con
     }
     const dim3 grid(M, (H + MOE_ROWS - 1) / MOE_ROWS);
     if (dtype == PTA_F32)
-        hipLaunchKernelGGL(moe_down_kernel<float>, grid, dim3(256), (size_t)top * F * 4, s, (float*)out, (const float*)act_in, (const float*)down, ids, wts, H, F, top);
+        hipLaunchKernelGGL(moe_down_kernel<float>, grid, dim3(256), (size_t)top * F * 4, s, (float*)out, (const float*)act_in, (const float*)down, ids, wts, H, F, top, (const float*)extra, extra_gate, gate_ld);
     else
-        hipLaunchKernelGGL(moe_down_kernel<bf16_t>, grid, dim3(256), (size_t)top * F * 4, s, (bf16_t*)out, (const bf16_t*)act_in, (const bf16_t*)down, ids, wts, H, F, top);
+        hipLaunchKernelGGL(moe_down_kernel<bf16_t>, grid, dim3(256), (size_t)top * F * 4, s, (bf16_t*)out, (const bf16_t*)act_in, (const bf16_t*)down, ids, wts, H, F, top, (const bf16_t*)extra, extra_gate, gate_ld);
     return pta_check_launch("moe_down");
 }
 
@@ -422,6 +473,42 @@ __global__ __launch_bounds__(256) void moe_grouped_up_kernel(bf16_t* __restrict_
     }
 }
 
+// The same for experts without a gate: act_sorted[slot, f] = act(U_e x).  A wave owns four groups of sixteen rows f of the
+// expert's one input matrix, a workgroup 256 rows.
+__global__ __launch_bounds__(256) void moe_grouped_up_plain_kernel(bf16_t* __restrict__ act_sorted, const bf16_t* __restrict__ x,
+                                                                   long x_ld, const bf16_t* __restrict__ up,
+                                                                   const int* __restrict__ sorted_pair,
+                                                                   const int* __restrict__ tile_expert, int H, int F, int top,
+                                                                   int act, int tiles) {
+    __shared__ __attribute__((aligned(16))) bf16_t lds[2 * MOE_TILE * MOE_XROW];
+    int tile, fb;
+    if (!moe_item(tiles, (F + 255) / 256, &tile, &fb)) return;
+    const int e = tile_expert[tile];
+    if (e < 0) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, gq = lane >> 4;
+    const int f0 = fb * 256 + wave * 64;
+    const bf16_t* arow[4];
+#pragma unroll
+    for (int a = 0; a < 4; ++a) arow[a] = up + ((long)e * F + min(f0 + a * 16 + c, F - 1)) * H + gq * 8;
+    const int pair = sorted_pair[tile * MOE_TILE + (tid >> 2)];
+    const bf16_t* brow = x + (long)(pair < 0 ? 0 : pair / top) * x_ld + (tid & 3) * 8;
+    moe_f32x4_t acc[4][4];
+    moe_tile_products<4>(acc, arow, brow, H, lds);
+    if (f0 >= F) return;
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+        const long slot = (long)tile * MOE_TILE + tt * 16 + c;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            float y[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) y[j] = apply_act(round_to_bf16(acc[a][tt][j]), act);
+            const int f = f0 + a * 16 + 4 * gq;
+            moe_store4(act_sorted + slot * F + f, f, F, y[0], y[1], y[2], y[3]);
+        }
+    }
+}
+
 // y_sorted[slot, n] = D_e act_sorted[slot]: a wave owns four groups of sixteen rows n of the expert's down matrix, a
 // workgroup 256 rows, against the tile's 64 slots
 __global__ __launch_bounds__(256) void moe_grouped_down_kernel(bf16_t* __restrict__ y_sorted, const bf16_t* __restrict__ act_sorted,
@@ -454,12 +541,14 @@ __global__ __launch_bounds__(256) void moe_grouped_down_kernel(bf16_t* __restric
 
 // out[m, n] = sum_k wts[m, k] * y_sorted[slot_of_pair[m * top + k], n], in the order the experts were taken
 __global__ void moe_combine_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ y_sorted,
-                                   const int* __restrict__ slot_of_pair, const float* __restrict__ wts, int H, int top) {
+                                   const int* __restrict__ slot_of_pair, const float* __restrict__ wts, int H, int top,
+                                   const bf16_t* __restrict__ extra, const float* __restrict__ extra_gate, int gate_ld) {
     const int m = blockIdx.x;
     for (int n = threadIdx.x; n < H; n += blockDim.x) {
         float acc = 0.f;
         for (int k = 0; k < top; ++k)
             acc += wts[(long)m * top + k] * bf16_bits_to_f32(y_sorted[(long)slot_of_pair[(long)m * top + k] * H + n]);
+        if (extra) acc += extra_gate[(long)m * gate_ld] * bf16_bits_to_f32(extra[(long)m * H + n]);
         out[(long)m * H + n] = f32_to_bf16_bits(acc);
     }
 }
@@ -471,7 +560,8 @@ extern "C" int pta_moe_grouped_slots(int pairs, int E) { return (pairs + E * (MO
 extern "C" int pta_moe_grouped(void* out, const void* x, long x_ld, const void* gate_up, const void* down, const int* ids,
                                const float* wts, int* sorted_pair, int* slot_of_pair, int* tile_expert, void* act_sorted,
                                void* y_sorted, int M, int H, int F, int E, int top, int act, const PtaGate* gate_how,
-                               void* stream) {
+                               int gated, const void* extra, const float* extra_gate, int gate_ld, void* stream) {
+    PTA_REQUIRE((extra != nullptr) == (extra_gate != nullptr), "moe_grouped: a further term and its gate come together");
     const PtaGate gate = gate_how ? *gate_how : PtaGate{PTA_GLU_SILU, 1.f, 0.f};
     PTA_REQUIRE(gate.kind == PTA_GLU_SILU || gate.kind == PTA_GLU_CLAMPED, "moe_grouped: a gate of kind %d is not built", gate.kind);
     PTA_REQUIRE(M > 0 && H > 0 && F > 0 && E > 0 && top > 0, "moe_grouped: sizes must be positive");
@@ -489,10 +579,15 @@ extern "C" int pta_moe_grouped(void* out, const void* x, long x_ld, const void* 
     hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), (size_t)(3 * E + 1) * 4, s, sorted_pair, slot_of_pair, tile_expert,
                        ids, (int)pairs, E, slots, tiles);
     auto grid_for = [&](int blocks) { return dim3((unsigned)(((long)tiles * blocks + 7) / 8 * 8)); };
-    hipLaunchKernelGGL(moe_grouped_up_kernel, grid_for((F + 127) / 128), dim3(256), 0, s, (bf16_t*)act_sorted, (const bf16_t*)x,
-                       x_ld, (const bf16_t*)gate_up, sorted_pair, tile_expert, H, F, top, act, gate, tiles);
+    if (gated)
+        hipLaunchKernelGGL(moe_grouped_up_kernel, grid_for((F + 127) / 128), dim3(256), 0, s, (bf16_t*)act_sorted, (const bf16_t*)x,
+                           x_ld, (const bf16_t*)gate_up, sorted_pair, tile_expert, H, F, top, act, gate, tiles);
+    else
+        hipLaunchKernelGGL(moe_grouped_up_plain_kernel, grid_for((F + 255) / 256), dim3(256), 0, s, (bf16_t*)act_sorted,
+                           (const bf16_t*)x, x_ld, (const bf16_t*)gate_up, sorted_pair, tile_expert, H, F, top, act, tiles);
     hipLaunchKernelGGL(moe_grouped_down_kernel, grid_for((H + 255) / 256), dim3(256), 0, s, (bf16_t*)y_sorted,
                        (const bf16_t*)act_sorted, (const bf16_t*)down, tile_expert, H, F, tiles);
-    hipLaunchKernelGGL(moe_combine_kernel, dim3(M), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)y_sorted, slot_of_pair, wts, H, top);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(M), dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)y_sorted, slot_of_pair, wts, H, top,
+                       (const bf16_t*)extra, extra_gate, gate_ld);
     return pta_check_launch("moe_grouped");
 }

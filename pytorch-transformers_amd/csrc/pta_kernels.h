@@ -271,7 +271,8 @@ int pta_ssm_scan(float* y, const float* xbc, const void* dt_in, long dt_ld, cons
 
 // ---- attention over a cache of latents (attn_latent.hip) ----------------------------------------------------------
 int pta_attn_latent_sizes_ok(int H, int dn, int dr, int R);
-int pta_latent_prep(float* q_full, void* k_pool, const void* proj, long ld, const float* w_norm, float eps,
+int pta_latent_prep(float* q_full, void* k_pool, const void* q_rows, long q_ld, const void* down_rows, long ld,
+                    const float* w_norm, float eps,
                     const PtaRotation* rot, const int* token_pos, const int* token_seq, const int* block_table,
                     int bt_stride, int M, int H, int dn, int dr, int R, int write_cache, int dtype, void* stream);
 int pta_head_project(void* out, int out_wide, long out_ld, long out_head, const void* in, int in_wide, long in_ld,
@@ -308,7 +309,9 @@ typedef struct PtaGate {
 // sqrt(mean over the row of v^2 + eps), and (a, b, c, e) the four 32-bit numbers of `coef`; sums in 32-bit.
 int pta_polynorm(void* out, const void* z, long z_ld, const float* coef, float eps, int M, int F, int dtype, void* stream);
 int pta_gated_heads(void* out, const void* x, int x_f32, long x_ld, int x_head, const void* g, long g_ld, const float* w,
-                    float eps, int M, int heads, int dv, int dtype, void* stream);
+                    float eps, int M, int heads, int dv, int g_per_head, int dtype, void* stream);
+// xIELU of z [M, F] (rows z_ld apart) with the two learned numbers act[0], act[1] (32-bit): see gated.hip
+int pta_xielu(void* out, const void* z, long z_ld, int M, int F, const float* act, int dtype, void* stream);
 int pta_glu(void* out, const void* gate, const void* up, long in_ld, int M, int F, int kind, float alpha, float limit,
             int dtype, void* stream);
 
@@ -320,15 +323,18 @@ int pta_decay_scan(float* y, const void* q, const void* k, const void* v, long l
 // ---- routed experts (moe.hip) -----------------------------------------------------------------------------------------
 enum PtaRouteScore { PTA_ROUTE_SIGMOID = 0, PTA_ROUTE_SOFTMAX = 1 };
 int pta_moe_route(int* ids, float* wts, const void* h, long h_ld, const float* Wr, const float* br, int M, int H, int E,
-                  int top, int score_kind, int normalise, float scale, int dtype, void* stream);
+                  int top, int score_kind, int normalise, float scale, int groups, int keep, const float* extra,
+                  float* extra_out, int n_extra, int dtype, void* stream);
+// gated 0: experts without a gate, gate_up is their one input matrix [E, F, H] and an expert is down(act(up h))
 int pta_moe_up(void* act_out, const void* h, long h_ld, const void* gate_up, const int* ids, int M, int H, int F, int top,
-               int act, const PtaGate* gate_how, int dtype, void* stream);
+               int act, const PtaGate* gate_how, int gated, int dtype, void* stream);
 int pta_moe_down(void* out, const void* act_in, const void* down, const int* ids, const float* wts, int M, int H, int F,
-                 int top, int dtype, void* stream);
+                 int top, const void* extra, const float* extra_gate, int gate_ld, int dtype, void* stream);
 int pta_moe_grouped_slots(int pairs, int E);
 int pta_moe_grouped(void* out, const void* x, long x_ld, const void* gate_up, const void* down, const int* ids,
                     const float* wts, int* sorted_pair, int* slot_of_pair, int* tile_expert, void* act_sorted, void* y_sorted,
-                    int M, int H, int F, int E, int top, int act, const PtaGate* gate_how, void* stream);
+                    int M, int H, int F, int E, int top, int act, const PtaGate* gate_how, int gated, const void* extra,
+                    const float* extra_gate, int gate_ld, void* stream);
 
 // ---- LayerNorm around a 32-bit stream (ln_stream.hip) -------------------------------------------------------------------
 int pta_layernorm_stream(void* out_narrow, float* out_wide, const float* x, const void* y, long y_ld, const float* wy,
@@ -339,9 +345,14 @@ int pta_embed_pos(float* out, const void* table, const int* ids, const void* pos
                   int M, int H, int positions, int dtype, void* stream);
 
 // ---- attention whose heads' scores are capped and mixed before the softmax (attn_talk.hip) -----------------------------
+// head_scale [nh] (null: none): a head's scores are multiplied by its number before the cap.  weights_kind: the softmax
+// over the keys a token sees, or PTA_WEIGHTS_SIGMOID: a key's weight is sigmoid(score + head_bias[h]) (head_bias [nh],
+// null: 0), not normalised over the keys.
+enum PtaWeights { PTA_WEIGHTS_SOFTMAX = 0, PTA_WEIGHTS_SIGMOID = 1 };
 int pta_attn_talk(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table, int bt_stride,
                   const int* token_seq, const int* token_pos, const float* talk, float softcap, int M, int nh, int nkv, int d,
-                  float scale, int window, int chunk, int dtype, void* stream);
+                  float scale, int window, int chunk, const float* head_scale, const float* head_bias, int weights_kind,
+                  int dtype, void* stream);
 // The same on the matrix cores (bfloat16; attn_talk_mfma.hip): a step's tokens by sequence (cu_tokens, seq_start) as
 // pta_attn_mfma takes them; with one token per sequence the keys may be cut into n_splits ranges of split_size.
 int pta_attn_talk_mfma_supported(int nh, int nkv, int d);
@@ -349,7 +360,8 @@ int pta_attn_talk_prompt_ranges(int tiles, int keys_seen);  // runs into which a
 int pta_attn_talk_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                        int bt_stride, const int* cu_tokens, const int* seq_start, const float* talk, float softcap,
                        int n_seqs, int max_new, int M, int nh, int nkv, int d, float scale, int window, int chunk,
-                       int split_size, int n_splits, float* po, float* pm, float* pl, void* stream);
+                       int split_size, int n_splits, float* po, float* pm, float* pl, const float* head_scale,
+                       const float* head_bias, int weights_kind, void* stream);
 // Merge of the partial results of ranges of keys (attn_mfma.hip): out[row] = sum_s w_s po[row, s] / sum_s w_s pl[row, s],
 // w_s = 2^(pm[row, s] - max_s pm); a range whose pm is -inf is not read.
 int pta_attn_combine(void* out, const float* po, const float* pm, const float* pl, long rows, int d, int n_splits,

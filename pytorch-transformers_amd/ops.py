@@ -198,7 +198,7 @@ def _entry_cost(name: str, a) -> tuple:
         M, H, K, O = float(a[9]), a[10], a[11], a[12]
         return (H * K * O * (4.0 if a[13] == F32 else 2.0) + M * H * (K + O) * 4.0, 2.0 * M * H * K * O)
     if name == "pta_latent_prep":
-        return (float(a[11]) * val(3) * (4.0 if a[17] == F32 else 2.0), 0.0)
+        return (float(a[13]) * (a[14] * (a[15] + a[16]) + a[17] + a[16]) * (4.0 if a[19] == F32 else 2.0), 0.0)
     el = lambda code: 4.0 if code == F32 else 2.0
     if name == "pta_shift_norm":  # the stream in and out (32-bit), the terms in, the two norms out
         M, H, e = float(a[16]), float(a[17]), el(a[20])
@@ -209,15 +209,17 @@ def _entry_cost(name: str, a) -> tuple:
         M, e = float(a[16]), el(a[23])
         return (M * e * ((a[17] + a[18]) * (a[19] + a[21]) + a[18] * (a[20] + a[21])), 0.0)
     if name == "pta_gated_heads":
-        M, N, e = float(a[9]), float(a[10] * a[11]), el(a[12])
+        M, N, e = float(a[9]), float(a[10] * a[11]), el(a[13])
         return (M * N * ((4.0 if a[2] else e) + 2 * e), 0.0)
+    if name == "pta_xielu":
+        return (float(a[3]) * a[4] * 2 * el(a[6]), 0.0)
     if name == "pta_glu":
         return (float(a[4]) * a[5] * 3 * el(a[9]), 0.0)
     if name == "pta_decay_scan":  # q, k, v in, o out in 32-bit; two multiply-adds per state element and token
         M, heads, P, N, e = float(timing_hint.get("rows", 0)), a[12], a[13], a[14], el(a[18])
         return (M * heads * ((2 * N + P) * e + P * 4.0), 4.0 * M * heads * N * P)
     if name == "pta_moe_route":
-        return (float(a[6]) * a[7] * el(a[13]) + float(a[7]) * a[8] * 4.0, 2.0 * a[6] * a[7] * a[8])
+        return (float(a[6]) * a[7] * el(a[18]) + float(a[7]) * a[8] * 4.0, 2.0 * a[6] * a[7] * a[8])
     if name == "pta_layernorm_stream":  # what it reads and writes: the stream, a sublayer's output, a second tensor, the results
         M, H, e = float(a[14]), float(a[15]), el(a[16])
         return (M * H * ((given(2) + given(8) + given(1)) * 4.0 + (given(3) + given(0)) * e), 0.0)
@@ -226,16 +228,16 @@ def _entry_cost(name: str, a) -> tuple:
     if name == "pta_embed_pos":
         return (float(a[6]) * a[7] * (2.0 * el(a[9]) + 4.0), 0.0)
     if name == "pta_moe_up":  # at most every (token, expert) pair's matrices once, and no more than all experts'
-        M, H, Fe, top, e = float(a[5]), a[6], a[7], a[8], el(a[11])
+        M, H, Fe, top, e, mats = float(a[5]), a[6], a[7], a[8], el(a[12]), (2 if a[11] else 1)
         pairs = min(M * top, float(timing_hint.get("experts", M * top)))
-        return (pairs * 2 * Fe * H * e, 4.0 * M * top * Fe * H)
+        return (pairs * mats * Fe * H * e, 2.0 * mats * M * top * Fe * H)
     if name == "pta_moe_down":
-        M, H, Fe, top, e = float(a[5]), a[6], a[7], a[8], el(a[9])
+        M, H, Fe, top, e = float(a[5]), a[6], a[7], a[8], el(a[12])
         pairs = min(M * top, float(timing_hint.get("experts", M * top)))
         return (pairs * Fe * H * e, 2.0 * M * top * Fe * H)
     if name == "pta_moe_grouped":  # every expert's three matrices once; the arithmetic of the pairs
-        M, H, Fe, E, top = float(a[12]), a[13], a[14], a[15], a[16]
-        return (min(E, M * top) * 3.0 * Fe * H * 2.0, 6.0 * M * top * Fe * H)
+        M, H, Fe, E, top, mats = float(a[12]), a[13], a[14], a[15], a[16], (3.0 if a[19] else 2.0)
+        return (min(E, M * top) * mats * Fe * H * 2.0, 2.0 * mats * M * top * Fe * H)
     return (0.0, 0.0)
 
 
@@ -326,12 +328,14 @@ def embed_pos(table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0, pos_ta
 
 def layernorm_stream(dtype: torch.dtype, *, x: Optional[torch.Tensor] = None, y: Optional[torch.Tensor] = None,
                      post=None, mult: float = 1.0, add: Optional[torch.Tensor] = None, vec: Optional[torch.Tensor] = None,
-                     pre=None, eps: float = 0.0, rows: Optional[torch.Tensor] = None, want_wide: bool = True):
+                     pre=None, eps: float = 0.0, rows: Optional[torch.Tensor] = None, want_wide: bool = True,
+                     want_narrow: bool = False):
     """LayerNorm around a stream held in 32-bit, one launch: ``s = x + mult * LN_post(y) + add + vec`` (each term if
     given: ``x``, ``add`` ``[tokens, H]`` 32-bit, ``y`` ``[tokens, H]`` in ``dtype`` with rows that may lie apart, ``vec``
     ``[H]`` 32-bit, ``post = (weight, bias)``), then ``LN_pre(s)`` in ``dtype`` if ``pre = (weight, bias)`` is given.
     LN is ``(v - mean) / sqrt(var + eps) * weight + bias`` with the biased variance.  ``rows`` takes those rows of the
-    inputs alone.  Returns ``(narrow or None, s or None)``; s is returned only if ``want_wide``."""
+    inputs alone.  Without ``pre``, ``want_narrow`` asks for s itself in ``dtype`` beside the 32-bit one (what the next
+    matrix product reads).  Returns ``(narrow or None, s or None)``; s is returned only if ``want_wide``."""
     ref = x if x is not None else y
     if ref is None:
         raise KernelError("layernorm_stream needs a stream or a sublayer's output")
@@ -360,7 +364,7 @@ def layernorm_stream(dtype: torch.dtype, *, x: Optional[torch.Tensor] = None, y:
     else:
         M = ref.shape[0]
     wide = torch.empty((M, H), dtype=torch.float32, device=ref.device) if (want_wide or pre is None) else None
-    narrow = torch.empty((M, H), dtype=dtype, device=ref.device) if pre is not None else None
+    narrow = torch.empty((M, H), dtype=dtype, device=ref.device) if (pre is not None or want_narrow) else None
     if M:
         _call("pta_layernorm_stream", _ptr(narrow), _ptr(wide), _ptr(x), _ptr(y), ctypes.c_long(y_ld),
               _ptr(post[0]) if y is not None else None, _ptr(post[1]) if y is not None else None, ctypes.c_float(mult),
@@ -557,11 +561,26 @@ def attn_talk_sizes_problem(nh: int, nkv: int, d: int) -> Optional[str]:
     return None
 
 
+WEIGHTS_CODES = {"softmax": 0, "sigmoid": 1}
+
+
+def _head_numbers(nh: int, head_scale, head_bias, weights: str):
+    if weights not in WEIGHTS_CODES:
+        raise KernelError(f"attention weights of kind {weights!r} are not built; built: {sorted(WEIGHTS_CODES)}")
+    for name, t in (("head_scale", head_scale), ("head_bias", head_bias)):
+        if t is not None:
+            _need(t, name, torch.float32, (nh,))
+    return _ptr(head_scale), _ptr(head_bias), WEIGHTS_CODES[weights]
+
+
 def attn_talk(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_pos, scale: float, *,
-              talk: Optional[torch.Tensor] = None, softcap: float = 0.0, window: int = 0, chunk: int = 0):
-    """Causal attention as ``attn_generic`` (no bias) whose scores are, before the softmax, capped (``softcap *
-    tanh(score / softcap)`` if ``softcap`` > 0) and mixed over the heads (``score_h <- sum_g talk[h, g] score_g`` if
-    ``talk`` ``[nh, nh]`` 32-bit is given); 32-bit arithmetic; out [M, nh*d]."""
+              talk: Optional[torch.Tensor] = None, softcap: float = 0.0, window: int = 0, chunk: int = 0,
+              head_scale: Optional[torch.Tensor] = None, head_bias: Optional[torch.Tensor] = None, weights: str = "softmax"):
+    """Causal attention as ``attn_generic`` (no bias) whose scores are, before the softmax, multiplied by a number per
+    head (``head_scale`` ``[nh]`` 32-bit), capped (``softcap * tanh(score / softcap)`` if ``softcap`` > 0) and mixed over
+    the heads (``score_h <- sum_g talk[h, g] score_g`` if ``talk`` ``[nh, nh]`` 32-bit is given).  ``weights``
+    ``"sigmoid"``: a key's weight is ``sigmoid(score + head_bias[h])``, not normalised over the keys, in place of the
+    softmax.  32-bit arithmetic; out [M, nh*d]."""
     _need(q, "q")
     M, nh, d = q.shape
     nkv = k_pool.shape[1]
@@ -575,7 +594,7 @@ def attn_talk(q: torch.Tensor, k_pool, v_pool, block_table, token_seq, token_pos
     if M:
         _call("pta_attn_talk", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), block_table.shape[1],
               _ptr(token_seq), _ptr(token_pos), _ptr(talk), ctypes.c_float(softcap), M, nh, nkv, d, ctypes.c_float(scale),
-              int(window), int(chunk), dtype_code(q.dtype), _stream())
+              int(window), int(chunk), *_head_numbers(nh, head_scale, head_bias, weights), dtype_code(q.dtype), _stream())
     return out
 
 
@@ -690,7 +709,8 @@ def attn_talk_mfma_ok(q: torch.Tensor, nkv: int) -> bool:
 
 def attn_talk_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start, scale: float, *, max_new: int,
                    talk: Optional[torch.Tensor] = None, softcap: float = 0.0, window: int = 0, chunk: int = 0,
-                   n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS) -> torch.Tensor:
+                   n_splits: int = 1, split_size: int = ATTN_SPLIT_KEYS, head_scale: Optional[torch.Tensor] = None,
+                   head_bias: Optional[torch.Tensor] = None, weights: str = "softmax") -> torch.Tensor:
     """``attn_talk`` on the matrix cores (bfloat16 in, 32-bit scores, mix and softmax); out [M, nh*d].  ``max_new``
     bounds the new tokens of any sequence of the step; with one token per sequence and ``n_splits`` > 1 the keys are
     cut into ranges of ``split_size`` (``n_splits * split_size`` bounds every context), merged by a second launch;
@@ -714,7 +734,7 @@ def attn_talk_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_
     _call("pta_attn_talk_mfma", _ptr(out), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(block_table), block_table.shape[1],
           _ptr(cu_tokens), _ptr(seq_start), _ptr(talk), ctypes.c_float(softcap), n_seqs, int(max_new), M, nh, nkv, d,
           ctypes.c_float(scale), int(window), int(chunk), int(split_size), int(n_splits), _ptr(po), _ptr(pm), _ptr(pl),
-          _stream())
+          *_head_numbers(nh, head_scale, head_bias, weights), _stream())
     return out
 
 
@@ -736,7 +756,7 @@ def talk_decode_ranges(n_seqs: int, max_len: int, window: int = 0, chunk: int = 
 
 
 def attention_talk(q: torch.Tensor, k_pool, v_pool, block_table, ctx, scale: float, *, talk=None, softcap: float = 0.0,
-                   window: int = 0, chunk: int = 0) -> torch.Tensor:
+                   window: int = 0, chunk: int = 0, head_scale=None, head_bias=None, weights: str = "softmax") -> torch.Tensor:
     """Attention of a step's tokens over the cache with capped scores that are mixed over the heads before the
     softmax: picks the kernel for the step's shape and type.  bfloat16 with sizes the matrix-core kernel is built
     for: that kernel, with the context cut into ranges when every sequence brings one token; anything else: the
@@ -751,9 +771,10 @@ def attention_talk(q: torch.Tensor, k_pool, v_pool, block_table, ctx, scale: flo
             n_splits, size = int(load_library().pta_attn_talk_prompt_ranges(tiles, seen)), 0
         return attn_talk_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, scale,
                               max_new=max(ctx.new_tokens), talk=talk, softcap=softcap, window=window, chunk=chunk,
-                              n_splits=n_splits, split_size=size)
+                              n_splits=n_splits, split_size=size, head_scale=head_scale, head_bias=head_bias,
+                              weights=weights)
     return attn_talk(q, k_pool, v_pool, block_table, ctx.token_seq, ctx.token_pos, scale, talk=talk, softcap=softcap,
-                     window=window, chunk=chunk)
+                     window=window, chunk=chunk, head_scale=head_scale, head_bias=head_bias, weights=weights)
 
 
 def sample(logits: torch.Tensor, *, do_sample: bool, temperature: float = 1.0, top_k: int = 0, top_p: float = 1.0,
@@ -1484,14 +1505,21 @@ def latent_sizes_problem(heads: int, dim: int, rot_dim: int, rank: int) -> Optio
 
 def latent_prep(proj: torch.Tensor, w_norm: torch.Tensor, eps: float, inv_freq, cs_scale: float, rotary_dim, pairing: str,
                 token_pos, token_seq, block_table, k_pool, heads: int, dim: int, rot_dim: int, rank: int,
-                write_cache: bool = True) -> torch.Tensor:
-    """From ``proj`` ``[tokens, heads * (dim + rot_dim) + rank + rot_dim]`` (the queries, then the down-projection):
-    the normed latent and the rotated shared key part go into the token's cache row ``[rank + rot_dim]``; returns
-    the queries' frame ``[tokens, heads, rank + rot_dim]`` in 32-bit with the rotated parts filled in (the first
-    ``rank`` of each head are for ``head_project``)."""
+                write_cache: bool = True, q: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """From ``proj`` ``[tokens, heads * (dim + rot_dim) + rank + rot_dim]`` (the queries, then the down-projection), or
+    with the queries ``q`` ``[tokens, heads * (dim + rot_dim)]`` given apart from ``proj`` ``[tokens, rank + rot_dim]``
+    (each may be a block of columns): the normed latent and the rotated shared key part go into the token's cache row
+    ``[rank + rot_dim]``; returns the queries' frame ``[tokens, heads, rank + rot_dim]`` in 32-bit with the rotated
+    parts filled in (the first ``rank`` of each head are for ``head_project``)."""
     M = proj.shape[0]
-    cols = heads * (dim + rot_dim) + rank + rot_dim
-    ld = _rows_of(proj, "proj", cols)
+    q_cols = heads * (dim + rot_dim)
+    if q is None:
+        ld = _rows_of(proj, "proj", q_cols + rank + rot_dim)
+        q_ptr, q_ld, down_ptr = proj.data_ptr(), ld, proj.data_ptr() + q_cols * proj.element_size()
+    else:
+        ld = _rows_of(proj, "proj", rank + rot_dim)
+        q_ld = _rows_of(q, "q", q_cols, proj.dtype)
+        q_ptr, down_ptr = q.data_ptr(), proj.data_ptr()
     _need(w_norm, "w_norm", torch.float32, (rank,))
     _need(token_pos, "token_pos", torch.int32, (M,))
     _need(token_seq, "token_seq", torch.int32, (M,))
@@ -1503,7 +1531,8 @@ def latent_prep(proj: torch.Tensor, w_norm: torch.Tensor, eps: float, inv_freq, 
     rot = _rotation_arg(inv_freq, cs_scale, rot_dim, block_table.shape[0], rotary_dim, pairing) if rot_dim else None
     q_full = torch.empty((M, heads, D), dtype=torch.float32, device=proj.device)
     if M:
-        _call("pta_latent_prep", _ptr(q_full), _ptr(k_pool), _ptr(proj), ctypes.c_long(ld), _ptr(w_norm),
+        _call("pta_latent_prep", _ptr(q_full), _ptr(k_pool), ctypes.c_void_p(q_ptr), ctypes.c_long(q_ld),
+              ctypes.c_void_p(down_ptr), ctypes.c_long(ld), _ptr(w_norm),
               ctypes.c_float(eps), rot, _ptr(token_pos), _ptr(token_seq), _ptr(block_table), block_table.shape[1], M,
               heads, dim, rot_dim, rank, int(write_cache), dtype_code(proj.dtype), _stream())
     return q_full
@@ -1684,20 +1713,34 @@ GLU_CODES = {"silu": 0, "clamped": 1}
 
 
 def gated_heads(x: torch.Tensor, x_head: int, g: torch.Tensor, heads: int, dv: int, dtype: torch.dtype,
-                w: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
+                w: Optional[torch.Tensor] = None, eps: float = 0.0, per_head: bool = False) -> torch.Tensor:
     """``n(x) * sigmoid(g)`` ``[M, heads * dv]`` in ``dtype``: ``x`` (32-bit or ``dtype``) holds heads of ``dv``
     elements in frames ``x_head`` apart; n is an RMS norm over the row of all heads with the weight ``w``, or the
-    identity (``w`` None); ``g`` ``[M, heads * dv]`` (``dtype``) may be a block of columns."""
+    identity (``w`` None); ``g`` ``[M, heads * dv]`` (``dtype``) may be a block of columns.  ``per_head``: the gate is
+    one number a head, ``g`` ``[M, heads]``."""
     M = x.shape[0]
     if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < (heads - 1) * x_head + dv or x.dtype not in (torch.float32, dtype):
         raise KernelError(f"x must be [M, at least {(heads - 1) * x_head + dv}] in 32-bit or {dtype}")
-    g_ld = _rows_of(g, "g", heads * dv, dtype)
+    g_ld = _rows_of(g, "g", heads if per_head else heads * dv, dtype)
     if w is not None:
         _need(w, "w", torch.float32, (heads * dv,))
     out = torch.empty((M, heads * dv), dtype=dtype, device=x.device)
     if M:
         _call("pta_gated_heads", _ptr(out), _ptr(x), int(x.dtype == torch.float32), ctypes.c_long(x.stride(0)), int(x_head),
-              _ptr(g), ctypes.c_long(g_ld), _ptr(w), ctypes.c_float(eps), M, heads, dv, dtype_code(dtype), _stream())
+              _ptr(g), ctypes.c_long(g_ld), _ptr(w), ctypes.c_float(eps), M, heads, dv, int(bool(per_head)), dtype_code(dtype),
+              _stream())
+    return out
+
+
+def xielu(z: torch.Tensor, act: torch.Tensor) -> torch.Tensor:
+    """xIELU element by element: with ``ap = softplus(act[0])`` and ``an = 1/2 + softplus(act[1])`` (``act``: two learned
+    numbers, 32-bit), ``ap z^2 + z / 2`` for z > 0 and ``an (e^z - 1 - z) + z / 2`` else; ``z`` may be a block of columns."""
+    M, F = z.shape
+    ld = _rows_of(z, "z", F)
+    _need(act, "act", torch.float32, (2,))
+    out = torch.empty((M, F), dtype=z.dtype, device=z.device)
+    if M:
+        _call("pta_xielu", _ptr(out), _ptr(z), ctypes.c_long(ld), M, F, _ptr(act), dtype_code(z.dtype), _stream())
     return out
 
 
@@ -1754,10 +1797,13 @@ ROUTE_SCORE_CODES = {"sigmoid": 0, "softmax": 1}
 
 
 def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, score: str = "sigmoid", normalise: bool = True,
-              scale: float = 1.0, bias: Optional[torch.Tensor] = None):
+              scale: float = 1.0, bias: Optional[torch.Tensor] = None, groups: int = 1, keep: int = 1,
+              extra: Optional[torch.Tensor] = None):
     """Per token the ``top`` experts with the largest scores of ``router @ h`` (+ ``bias``; 32-bit; ``router``
     ``[experts, features]`` and ``bias`` ``[experts]`` 32-bit) and their weights: ``(ids [M, top] int32, weights [M,
-    top] 32-bit)``."""
+    top] 32-bit)``.  With ``groups`` > 1 the experts form that many equal runs of neighbours, a run's score is its
+    largest, and only experts of the ``keep`` best runs can be taken.  ``extra`` ``[rows, features]`` (32-bit): the
+    launch also forms ``sigmoid(extra @ h)`` ``[M, rows]`` in 32-bit, returned as a third value."""
     M, H = h.shape
     E = router.shape[0]
     _need(router, "router", torch.float32, (E, H))
@@ -1766,33 +1812,46 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, top: int, score: str = "sig
     ld = _rows_of(h, "h", H)
     ids = torch.empty((M, top), dtype=torch.int32, device=h.device)
     wts = torch.empty((M, top), dtype=torch.float32, device=h.device)
+    gates, X = None, 0
+    if extra is not None:
+        X = extra.shape[0]
+        _need(extra, "extra", torch.float32, (X, H))
+        gates = torch.empty((M, X), dtype=torch.float32, device=h.device)
     if M:
         _call("pta_moe_route", _ptr(ids), _ptr(wts), _ptr(h), ctypes.c_long(ld), _ptr(router), _ptr(bias), M, H, E, int(top),
-              ROUTE_SCORE_CODES[score], int(bool(normalise)), ctypes.c_float(scale), dtype_code(h.dtype), _stream())
-    return ids, wts
+              ROUTE_SCORE_CODES[score], int(bool(normalise)), ctypes.c_float(scale), int(groups), int(keep), _ptr(extra),
+              _ptr(gates), int(X), dtype_code(h.dtype), _stream())
+    return (ids, wts) if extra is None else (ids, wts, gates)
 
 
 MOE_GROUPED_FROM_ROWS = 16  # steps of more tokens run their experts on the matrix cores (bfloat16)
 
 
 def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor,
-                act: str = "silu", gate=None) -> torch.Tensor:
+                act: str = "silu", gate=None, gated: bool = True, extra: Optional[torch.Tensor] = None,
+                extra_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``sum_k wts[m, k] * down[e] (act(gate[e] h) * (up[e] h))`` with ``e = ids[m, k]``: ``gate_up`` ``[experts, 2 F,
     features]`` (an expert's gate rows, then its up rows), ``down`` ``[experts, features, F]``; out ``[M, features]``.
     ``gate = (kind, alpha, limit)`` of ``GLU_CODES``: with ``"clamped"`` an expert's two products meet as ``glu`` says
-    in place of ``act(g) * u``."""
+    in place of ``act(g) * u``.  ``gated=False``: experts without a gate, ``down[e] act(up[e] h)``, with ``gate_up`` their
+    one input matrix ``[experts, F, features]``.  ``extra`` ``[M, features]`` with ``extra_gate`` ``[M, 1]`` (32-bit, rows
+    may lie apart): ``extra_gate[m] * extra[m]`` is added in the launch that sums the experts."""
     how = None
     if gate is not None:
         how = ctypes.byref(_PtaGate(GLU_CODES[gate[0]], float(gate[1]), float(gate[2])))
     M, H = h.shape
     E, F2, _ = gate_up.shape
-    F = F2 // 2
+    F = F2 // 2 if gated else F2
     top = ids.shape[1]
-    _need(gate_up, "gate_up", h.dtype, (E, 2 * F, H))
+    _need(gate_up, "gate_up", h.dtype, (E, (2 if gated else 1) * F, H))
     _need(down, "down", h.dtype, (E, H, F))
     _need(ids, "ids", torch.int32, (M, top))
     _need(wts, "wts", torch.float32, (M, top))
     ld = _rows_of(h, "h", H, h.dtype)
+    gate_ld = 0
+    if extra is not None:
+        _need(extra, "extra", h.dtype, (M, H))
+        gate_ld = _rows_of(extra_gate, "extra_gate", 1, torch.float32)
     out = torch.empty((M, H), dtype=h.dtype, device=h.device)
     timing_hint["experts"] = E
     if (h.dtype == torch.bfloat16 and M > MOE_GROUPED_FROM_ROWS and H % 64 == 0 and F % 64 == 0 and ld % 8 == 0
@@ -1804,12 +1863,13 @@ def moe_experts(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, ids:
         y_sorted = torch.empty((slots, H), dtype=h.dtype, device=h.device)
         _call("pta_moe_grouped", _ptr(out), _ptr(h), ctypes.c_long(ld), _ptr(gate_up), _ptr(down), _ptr(ids), _ptr(wts),
               _ptr(ints[:slots]), _ptr(ints[slots:slots + M * top]), _ptr(ints[slots + M * top:]), _ptr(act_sorted),
-              _ptr(y_sorted), M, H, F, E, top, ACT_CODES[act], how, _stream())
+              _ptr(y_sorted), M, H, F, E, top, ACT_CODES[act], how, int(bool(gated)), _ptr(extra), _ptr(extra_gate),
+              int(gate_ld), _stream())
         return out
     act_buf = torch.empty((M * top, F), dtype=h.dtype, device=h.device)
     if M:
         _call("pta_moe_up", _ptr(act_buf), _ptr(h), ctypes.c_long(ld), _ptr(gate_up), _ptr(ids), M, H, F, top,
-              ACT_CODES[act], how, dtype_code(h.dtype), _stream())
-        _call("pta_moe_down", _ptr(out), _ptr(act_buf), _ptr(down), _ptr(ids), _ptr(wts), M, H, F, top,
-              dtype_code(h.dtype), _stream())
+              ACT_CODES[act], how, int(bool(gated)), dtype_code(h.dtype), _stream())
+        _call("pta_moe_down", _ptr(out), _ptr(act_buf), _ptr(down), _ptr(ids), _ptr(wts), M, H, F, top, _ptr(extra),
+              _ptr(extra_gate), int(gate_ld), dtype_code(h.dtype), _stream())
     return out

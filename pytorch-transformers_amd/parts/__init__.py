@@ -4,7 +4,7 @@ from .linear import Embedding, Linear, OutputHead, QkvTail, TailDone
 from .norms import LayerNorm, RMSNorm
 from .positions import AlibiPositions, NoPositions, Rotation, RotaryPositions, ScoreBias, alibi_slopes
 from .attention import AttentionMixer
-from .feedforward import DenseFeedForward, GatedFeedForward, PolyNormFeedForward, RoutedFeedForward
+from .feedforward import DenseFeedForward, GatedFeedForward, PolyNormFeedForward, RoutedFeedForward, XieluFeedForward
 from .blocks import ParallelBlock, PostNormBlock, SandwichBlock, SequentialBlock, ShiftedParallelBlock
 from .gated_attention import GatedAttentionMixer
 from .linear_attention import DecayLinearAttentionMixer
@@ -17,4 +17,4 @@ __all__ = ["Part", "StepContext", "make_part", "register_part", "registered_part
            "AttentionMixer", "DenseFeedForward", "ParallelBlock", "SequentialBlock", "PostNormBlock", "RMSNorm", "DepthMix",
            "LatentAttentionMixer", "GatedScanMixer", "StateSpaceMixer", "GatedFeedForward", "RoutedFeedForward",
            "ShiftedParallelBlock", "GatedAttentionMixer", "DecayLinearAttentionMixer", "SandwichBlock", "LoopEntry",
-           "PolyNormFeedForward"]
+           "PolyNormFeedForward", "XieluFeedForward"]

@@ -71,6 +71,32 @@ class PolyNormFeedForward(Part):
         return self.down(y, add1=as_tensor(add1), add2=as_tensor(add2))
 
 
+class XieluFeedForward(Part):
+    """``down(act(up(x)))`` without biases, with the activation xIELU: with two learned numbers (p, q) and ``ap =
+    softplus(p)``, ``an = 1/2 + softplus(q)``, element by element ``ap z^2 + z / 2`` for z > 0 and ``an (e^z - 1 - z) +
+    z / 2`` else.  The two softplus and the activation are 32-bit.  The file holds ``name.up``, ``name.down`` and the two
+    numbers as ``name.act``."""
+
+    def __init__(self, name: str, hidden_size: int, ffn_size: int):
+        self.name, self.ffn_size = name, int(ffn_size)
+        self.up = Linear(f"{name}.up", hidden_size, ffn_size, False, weight_name=f"{name}.up")
+        self.down = Linear(f"{name}.down", ffn_size, hidden_size, False, weight_name=f"{name}.down")
+        self.coef: Optional[torch.Tensor] = None
+
+    def children(self) -> Sequence[Part]:
+        return (self.up, self.down)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(f"{self.name}.act", (2,), VECTOR, INIT_ZERO_NOISE)]
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.coef = tensors[f"{self.name}.act"]
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None):
+        y = ops.xielu(self.up(x), self.coef)
+        return self.down(y, add1=as_tensor(add1), add2=as_tensor(add2))
+
+
 class GatedFeedForward(Part):
     """A feed-forward with a gate: ``down(glu(gate(x), up(x)))``, no biases.  ``kind`` ``"silu"``: ``silu(gate) * up``;
     ``"clamped"``: with ``g = min(gate, limit)`` and ``u = clamp(up, -limit, limit)``, ``g * sigmoid(alpha * g) * (u +
@@ -136,12 +162,19 @@ class RoutedFeedForward(Part):
     expert's two input products meet as ``ops.glu`` of that kind says (``"clamped"``: ``g = min(gate, limit)``, ``u =
     clamp(up, -limit, limit)``, ``g * sigmoid(alpha g) * (u + 1)``) in place of ``act(gate) * up``.
 
+    ``gated=False``: experts without a gate, ``down_e(act(up_e x))``.  ``groups = (count, keep)``: the experts form
+    ``count`` equal groups of neighbours, a group's score is its largest s, and only experts of the ``keep`` best groups
+    can be taken.  ``shared_ff`` > 0: one more expert of that size (``name.shared.up``, ``.down``; same form, no gate)
+    runs for every token and is added, times ``sigmoid(W_sg x)`` (``name.shared.sg`` ``[1, hidden]``, one number a
+    token, formed in 32-bit by the router's launch) if ``shared_gate``.
+
     The file holds ``name.router`` ``[experts, hidden]`` and per expert ``name.e<j>.gate``, ``.up`` ``[ff, hidden]``
     and ``.down`` ``[hidden, ff]``; on the device the experts' matrices are stacked (gate rows then up rows per
     expert, and the down matrices) and the router is 32-bit."""
 
     def __init__(self, name: str, hidden_size: int, ffn_size: int, experts: int, top: int, scale: float = 1.0,
-                 score: str = "sigmoid", normalise: bool = True, act: str = "silu", router_bias: bool = False, gate=None):
+                 score: str = "sigmoid", normalise: bool = True, act: str = "silu", router_bias: bool = False, gate=None,
+                 gated: bool = True, groups=None, shared_ff: int = 0, shared_gate: bool = False):
         if gate is not None and gate[0] not in ops.GLU_CODES:
             raise ValueError(f"{name}: a gate of kind {gate[0]!r} is not built; built: {sorted(ops.GLU_CODES)}")
         if not (0 < top <= experts):
@@ -152,31 +185,62 @@ class RoutedFeedForward(Part):
         self.experts, self.top, self.scale = int(experts), int(top), float(scale)
         self.score, self.normalise, self.act = score, bool(normalise), act
         self.router_bias, self.gate = bool(router_bias), (None if gate is None else (gate[0], float(gate[1]), float(gate[2])))
-        self.router = self.gate_up = self.down = self.bias = None
+        self.gated = bool(gated)
+        if not self.gated and (gate is not None or act not in ops.ACT_CODES):
+            raise ValueError(f"{name}: experts without a gate take an activation of {sorted(k for k in ops.ACT_CODES if k)}")
+        self.groups = (1, 1) if groups is None else (int(groups[0]), int(groups[1]))
+        count, keep = self.groups
+        if count < 1 or experts % count or not (1 <= keep <= count) or keep * (experts // count) < top:
+            raise ValueError(f"{name}: {experts} experts in {count} groups of which {keep} are kept do not give {top} a token")
+        self.shared = None
+        self.shared_gate = bool(shared_gate) and shared_ff > 0
+        if shared_ff > 0:
+            self.shared = DenseFeedForward(f"{name}.shared", hidden_size, int(shared_ff), False, act, "up", "down",
+                                           bare_names=True)
+        self.router = self.gate_up = self.down = self.bias = self.shared_gate_w = None
+
+    def children(self) -> Sequence[Part]:
+        return () if self.shared is None else (self.shared,)
 
     def tensor_specs(self) -> List[TensorSpec]:
         n, E, F, H = self.name, self.experts, self.ffn_size, self.hidden_size
-        gu = tuple((f"{n}.e{e}.{m}", (F, H)) for e in range(E) for m in ("gate", "up"))
         dn = tuple((f"{n}.e{e}.down", (H, F)) for e in range(E))
         bias = [TensorSpec(f"{n}.router.b", (E,), VECTOR, INIT_ZERO_NOISE)] if self.router_bias else []
-        return bias + [TensorSpec(f"{n}.router", (E, H), VECTOR, INIT_NORMAL),
-                TensorSpec(f"{n}.experts.gate_up", (E, 2 * F, H), MATRIX, INIT_NORMAL, pieces=gu,
-                           assemble=_stack_experts(E, (F, F)), split=_unstack_experts((F, F))),
+        if self.shared_gate:
+            bias.append(TensorSpec(f"{n}.shared.sg", (1, H), VECTOR, INIT_NORMAL))
+        if self.gated:
+            gu = tuple((f"{n}.e{e}.{m}", (F, H)) for e in range(E) for m in ("gate", "up"))
+            first = TensorSpec(f"{n}.experts.gate_up", (E, 2 * F, H), MATRIX, INIT_NORMAL, pieces=gu,
+                               assemble=_stack_experts(E, (F, F)), split=_unstack_experts((F, F)))
+        else:
+            up = tuple((f"{n}.e{e}.up", (F, H)) for e in range(E))
+            first = TensorSpec(f"{n}.experts.up", (E, F, H), MATRIX, INIT_NORMAL, pieces=up,
+                               assemble=_stack_experts(E, (F,)), split=_unstack_experts((F,)))
+        return bias + [TensorSpec(f"{n}.router", (E, H), VECTOR, INIT_NORMAL), first,
                 TensorSpec(f"{n}.experts.down", (E, H, F), MATRIX, INIT_NORMAL, pieces=dn, assemble=_stack_experts(E, (H,)),
                            split=_unstack_experts((H,)))]
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         n = self.name
-        self.router, self.gate_up, self.down = tensors[f"{n}.router"], tensors[f"{n}.experts.gate_up"], tensors[f"{n}.experts.down"]
+        self.router, self.down = tensors[f"{n}.router"], tensors[f"{n}.experts.down"]
+        self.gate_up = tensors[f"{n}.experts.gate_up" if self.gated else f"{n}.experts.up"]
         self.bias = tensors[f"{n}.router.b"] if self.router_bias else None
+        self.shared_gate_w = tensors[f"{n}.shared.sg"] if self.shared_gate else None
 
     def check_sizes(self) -> None:
-        if self.top > 64 or self.experts > 2048:
-            raise ValueError(f"{self.name}: the router takes at most 64 of at most 2048 experts")
+        if self.top > 64 or self.experts > 2048 or self.groups[0] > 64:
+            raise ValueError(f"{self.name}: the router takes at most 64 of at most 2048 experts in at most 64 groups")
 
     def forward(self, x: torch.Tensor, ctx: StepContext, add1=None, add2=None):
-        ids, wts = ops.moe_route(x, self.router, self.top, self.score, self.normalise, self.scale, bias=self.bias)
-        out = ops.moe_experts(x, self.gate_up, self.down, ids, wts, self.act, gate=self.gate)
+        routed = ops.moe_route(x, self.router, self.top, self.score, self.normalise, self.scale, bias=self.bias,
+                               groups=self.groups[0], keep=self.groups[1], extra=self.shared_gate_w)
+        ids, wts = routed[0], routed[1]
+        extra = extra_gate = None
+        if self.shared is not None:  # the expert of every token: added, times its gate, by the launch that sums the taken ones
+            extra = self.shared.forward(x, ctx)
+            extra_gate = routed[2] if self.shared_gate else torch.ones((x.shape[0], 1), dtype=torch.float32, device=x.device)
+        out = ops.moe_experts(x, self.gate_up, self.down, ids, wts, self.act, gate=self.gate, gated=self.gated, extra=extra,
+                              extra_gate=extra_gate)
         if add1 is None and add2 is None:
             return out
         return ops.epilogue_(out, None, None, as_tensor(add1), as_tensor(add2))
@@ -185,4 +249,5 @@ class RoutedFeedForward(Part):
 register_part("feed_forward", "dense", DenseFeedForward)
 register_part("feed_forward", "gated", GatedFeedForward)
 register_part("feed_forward", "polynorm", PolyNormFeedForward)
+register_part("feed_forward", "xielu", XieluFeedForward)
 register_part("feed_forward", "routed", RoutedFeedForward)

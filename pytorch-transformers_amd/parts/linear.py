@@ -56,16 +56,28 @@ class Linear(Part):
         self.joined = None  # (both matrices as one, the other Linear) after ``join``
 
     @staticmethod
-    def stacked(name: str, layers: "Sequence[Linear]") -> "Linear":
-        """One layer whose rows are those of ``layers`` (loaded, one input size, no bias applied by it) one after
-        the other, for products of the same input that are to run as one.  The layers' own matrices become views of
-        the stacked one, so nothing is held twice; biases stay with the layers."""
+    def stacked(name: str, layers: "Sequence[Linear]", pad_to: int = 1, with_bias: bool = False) -> "Linear":
+        """One layer whose rows are those of ``layers`` (loaded, one input size) one after the other, for products of
+        the same input that are to run as one.  The layers' own matrices become views of the stacked one, so nothing
+        is held twice.  ``pad_to``: rows of zeros behind them, up to the next multiple, so that a result's rows start
+        at addresses that whoever reads blocks of its columns can load sixteen bytes from.  Biases stay with the layers
+        unless ``with_bias``: then the stacked layer applies them (zeros for a layer that has none)."""
         ws = [l.weight for l in layers]
         if any(w is None for w in ws) or len({(w.dtype, w.device, w.shape[1]) for w in ws}) != 1:
             raise ValueError(f"{name}: layers to stack must be loaded and agree in type, device and input size")
+        rows = sum(w.shape[0] for w in ws)
+        pad = -rows % max(int(pad_to), 1)
+        if pad:
+            ws = ws + [torch.zeros((pad, ws[0].shape[1]), dtype=ws[0].dtype, device=ws[0].device)]
         both = torch.cat(ws, dim=0).contiguous()
         out = Linear(name, ws[0].shape[1], both.shape[0], False)
         out.weight, out.bias, out.joined = both, None, None
+        if with_bias and any(l.bias is not None for l in layers):
+            ref = next(l.bias for l in layers if l.bias is not None)
+            parts = [l.bias if l.bias is not None else torch.zeros(l.out_features, dtype=ref.dtype, device=ref.device)
+                     for l in layers]
+            out.bias = torch.cat(parts + ([torch.zeros(pad, dtype=ref.dtype, device=ref.device)] if pad else [])).contiguous()
+            out.has_bias = True
         at = 0
         for l in layers:
             l.weight = both[at:at + l.out_features]

@@ -35,6 +35,19 @@ class LayerNorm(Part):
         """(weight, bias), for a launch that applies this norm beside other work (``ops.layernorm_stream``)."""
         return self.weight, self.bias
 
+    def apply(self, y: torch.Tensor, dtype: torch.dtype, *, residual: Optional[torch.Tensor] = None, mult: float = 1.0,
+              want_wide: bool = True, out_wide=None, mix=None):
+        """This norm on a sublayer's output ``y`` (compute type), times ``mult``, added to the 32-bit stream
+        ``residual``: ``(the new stream in dtype, the new stream in 32-bit)``, one launch (the interface of
+        ``RMSNorm.apply`` as far as a block whose norms stand on the sublayers' outputs uses it)."""
+        if out_wide is not None or mix is not None:
+            raise ValueError(f"{self.name}: a LayerNorm on a sublayer's output writes a stream of its own and mixes none")
+        if dtype == torch.float32:  # the stream is its own copy in the compute type
+            wide = ops.layernorm_stream(dtype, x=residual, y=y, post=self.affine(), mult=mult, eps=self.eps)[1]
+            return wide, wide
+        return ops.layernorm_stream(dtype, x=residual, y=y, post=self.affine(), mult=mult, eps=self.eps, want_wide=want_wide,
+                                    want_narrow=True)
+
     def forward_wide(self, x, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """The norm of a stream held in 32-bit (a ``WideResidual``), in its compute type.  A stream whose last
         sublayer is still to be normed and added (``PendingNormSum``) has that done in the same launch."""
