@@ -470,6 +470,40 @@ def kekapel_config(size, layers, vocab=32768):
                          residual_mult=0.7, initializer_range=0.02)
 
 
+# ---- the Nopuzen design beside the Kekapel and Pavodra models (--design nopuzen) ---------------------------------------
+NOPUZEN_SIZES = {
+    # width; the dense feed-forward (two matrices); latent attention heads (128 plain + 64 rotated elements, values of 128,
+    # latents of 512 for keys and values and 1,536 for queries); attention heads of 128 on 8 KV heads, scores capped at 30;
+    # 16 experts of two matrices in 4 groups of which 2 are kept and a token uses 2, together as large as the dense
+    # feed-forward, and a shared expert an eighth of it
+    "2k": dict(width=2048, ff=8192, heads=16, expert_ff=4096, shared_ff=1024),
+    "4k": dict(width=4096, ff=16384, heads=32, expert_ff=8192, shared_ff=2048),
+}
+NOPUZEN_KERNEL_LABELS = {
+    "pta_xielu": "xIELU between the dense feed-forward's two products",
+    "pta_gated_heads": "output gate (a number an element, or one a head)",
+    "pta_moe_grouped_up_plain": "experts' one input product on the matrix cores, tiles of one expert's tokens",
+}
+
+
+def nopuzen_config(size, layers, vocab=32768):
+    """Latent attention and attention with sigmoid weights in turn, dense and routed feed-forwards in turn."""
+    from pytorch_transformers_amd.config import NopuzenConfig
+
+    z = NOPUZEN_SIZES[size]
+    dense = {"kind": "dense", "ff": z["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": z["expert_ff"]}, "shared": {"ff": z["shared_ff"]},
+           "router": {"experts": 16, "top": 2, "scale": 1.0, "groups": {"count": 4, "keep": 2}}}
+    lat = {"heads": z["heads"], "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "q_rank": 1536, "scale": 192 ** -0.5,
+           "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+    attn = {"heads": z["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0,
+            "rot": {"base": 10000.0, "dims": 128}}
+    kinds = [{"type": "latent_attention", "mixer": lat, "mlp": dense}, {"type": "attention", "mixer": attn, "mlp": moe},
+             {"type": "latent_attention", "mixer": lat, "mlp": moe}, {"type": "attention", "mixer": attn, "mlp": dense}]
+    return NopuzenConfig(vocab=vocab, width=z["width"], layers=[kinds[i % 4] for i in range(layers)], norm={"eps": 1e-6},
+                         initializer_range=0.02)
+
+
 def falcon_like(size, layers, vocab=32768):
     """The closest model the library had: Falcon's new architecture at the same width, feed-forward, depth and
     vocabulary, heads of 128 in 8 groups."""
@@ -494,17 +528,23 @@ def design_record(args):
     KERNEL_LABELS.update(PAVODRA_KERNEL_LABELS)
     KERNEL_LABELS.update(BIMEPEL_KERNEL_LABELS)
     KERNEL_LABELS.update(KEKAPEL_KERNEL_LABELS)
+    KERNEL_LABELS.update(NOPUZEN_KERNEL_LABELS)
     design = args.design
-    design_config = {"pavodra": pavodra_config, "bimepel": bimepel_config, "kekapel": kekapel_config}[design]
+    configs = {"pavodra": pavodra_config, "bimepel": bimepel_config, "kekapel": kekapel_config, "nopuzen": nopuzen_config,
+               "falcon": falcon_like}
+    design_config = configs[design]
+    # the models a design stands beside: Falcon's, or for a design whose mechanisms came with other designs, those
+    beside = {"nopuzen": ("kekapel", "pavodra")}.get(design, ("falcon",))
     gen_cfg = GenerationConfig(do_sample=False, eos_token_id=None)
     layers, T, ctx_len = args.layers or 6, args.prefill_tokens, args.prompt_len
-    out = {"design": design, "beside": "falcon (new architecture, 8 KV groups of head size 128)", "dtype": args.dtype,
+    beside_text = "falcon (new architecture, 8 KV groups of head size 128)" if beside == ("falcon",) else ", ".join(beside)
+    out = {"design": design, "beside": beside_text, "dtype": args.dtype,
            "layers": layers, "prefill_tokens": T, "decode_context": ctx_len, "data": "synthetic token ids, random weights",
            "sizes": {}}
     dtype = "bfloat16" if args.dtype == "bf16" else "float32"
     for size in args.design_sizes.split(","):
         rec = {}
-        for name, cfg in ((design, design_config(size, layers)), ("falcon", falcon_like(size, layers))):
+        for name, cfg in [(design, design_config(size, layers))] + [(b, configs[b](size, layers)) for b in beside]:
             model = AutoModelForCausalLM.from_config(cfg, seed=0, dtype=dtype, device="cuda:0")
             r = {}
             pt = run_prefill(model, T)
@@ -520,9 +560,16 @@ def design_record(args):
                 cache = model.new_cache(b * ((ctx_len + 8 + page - 1) // page * page), max_slots=b)
                 slots = [cache.alloc() for _ in range(b)]
                 model.step(cache, slots, prompts, "last")
+                by_entry = {}
                 if name == "pavodra":
                     row, heads, rank = 576, PAVODRA_SIZES[size]["heads"], 512
                     kv, fl = b * (ctx_len + 1) * row * 2, 2.0 * heads * (row + rank) * T * (T + 1) / 2
+                elif name == "nopuzen":  # latent rows for one kind of layer, keys and values for the other
+                    row, heads, rank = 576, NOPUZEN_SIZES[size]["heads"], 512
+                    kv, fl = b * (ctx_len + 1) * row * 2, 2.0 * heads * (row + rank) * T * (T + 1) / 2
+                    a = cfg.layers[1]["mixer"]
+                    by_entry = {"attn_bytes:pta_attn_talk_mfma": b * (ctx_len + 1) * a["kv_heads"] * (a["dim"] + a["vdim"]) * 2,
+                                "attn_flops:pta_attn_talk_mfma": 2.0 * (a["dim"] + a["vdim"]) * a["heads"] * T * (T + 1) / 2}
                 elif name == "bimepel":  # keys and values of a token's own block of positions only
                     a = cfg.layers[0]["mixer"]
                     block = a["mask"]["size"]
@@ -538,6 +585,7 @@ def design_record(args):
                 else:
                     kv = b * (ctx_len + 1) * 2 * cfg.kv_heads * cfg.head_dim * 2
                     fl = 2.0 * cfg.head_dim * cfg.num_attention_heads * T * (T + 1)
+                ops.timing_hint.update(by_entry)
                 r["kernels_decode_b8"] = kernel_figures(model, ops, args.dtype, lambda: model.step(cache, slots, [[1]] * b, "last"),
                                                         attn_bytes=kv)
                 for s_ in slots:
@@ -552,6 +600,8 @@ def design_record(args):
                     cache.free(slot)
 
                 r[f"kernels_prefill_{T}"] = kernel_figures(model, ops, args.dtype, step, attn_flops=fl)
+                for key in by_entry:
+                    ops.timing_hint.pop(key, None)
                 del cache
             rec[name] = r
             del model
@@ -562,7 +612,7 @@ def design_record(args):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", default=None, choices=["pavodra", "bimepel", "kekapel"],
+    ap.add_argument("--design", default=None, choices=["pavodra", "bimepel", "kekapel", "nopuzen"],
                     help="measure that design beside the closest Falcon model at equal layer sizes and print that record "
                          "instead of the default run's (--layers, --prefill-tokens, --prompt-len and --dtype apply)")
     ap.add_argument("--design-sizes", default="2k,4k", help="with --design: which of the layer sizes 2k, 4k")

@@ -176,7 +176,9 @@ def _entry_cost(name: str, a) -> tuple:
         return ((a[4] + a[7]) * float(a[17]) * a[19] * 4, 0.0)
     if name in ("pta_attn_mfma", "pta_attn_generic", "pta_attn_latent_mfma", "pta_attn_latent", "pta_attn_talk",
                 "pta_attn_talk_mfma"):
-        return (float(timing_hint.get("attn_bytes", 0)), float(timing_hint.get("attn_flops", 0)))
+        # (a model with two kinds of attention says each kind's figures under the entry point's name)
+        return (float(timing_hint.get("attn_bytes:" + name, timing_hint.get("attn_bytes", 0))),
+                float(timing_hint.get("attn_flops:" + name, timing_hint.get("attn_flops", 0))))
     val = lambda i: float(getattr(a[i], "value", a[i]) or 0)
     given = lambda i: 1.0 if getattr(a[i], "value", a[i]) else 0.0
     if name == "pta_rmsnorm":  # what it reads and writes: x (and gate), the residual, the two results

@@ -65,8 +65,10 @@ def rotary_magnitude(rot: dict) -> float:
 
 def rotate(v: torch.Tensor, pos: int, rot: dict, layout: str) -> torch.Tensor:
     """The first ``dims`` elements of the last dimension turned by the position, the rest as they are.  Pairs: ``half``
-    (i, i + dims/2), ``interleaved`` (2i, 2i + 1); the pair (u, w) becomes (u cos a - w sin a, w cos a + u sin a), a =
+    (i, i + dims/2), ``interleaved`` (2i, 2i + 1); no ``rot``: nothing turns; the pair (u, w) becomes (u cos a - w sin a, w cos a + u sin a), a =
     pos * f_i, cos and sin times the magnitude."""
+    if not rot:
+        return v
     dims = int(rot["dims"])
     f = rotary_frequencies(rot)
     a = pos * f
@@ -114,7 +116,7 @@ def attention_token(w, p: str, m: dict, eps: float, h: torch.Tensor, kept: List,
     sigmoid(s + pb[g]), not normalised over j.  Head g's weighted sum of values, times sigmoid(W_g h)[g]; the heads side
     by side through W_o, plus b_o."""
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    rot = m["rot"]
+    rot = m.get("rot")
     q = (w[p + ".q"] @ h + w[p + ".q.b"]).view(H, d)
     k = (w[p + ".k"] @ h + w[p + ".k.b"]).view(G, d)
     v = (w[p + ".v"] @ h + w[p + ".v.b"]).view(G, dv)
