@@ -560,7 +560,7 @@ def design_record(args):
                 cache = model.new_cache(b * ((ctx_len + 8 + page - 1) // page * page), max_slots=b)
                 slots = [cache.alloc() for _ in range(b)]
                 model.step(cache, slots, prompts, "last")
-                by_entry = {}
+                by_entry, by_prompt = {}, {}
                 if name == "pavodra":
                     row, heads, rank = 576, PAVODRA_SIZES[size]["heads"], 512
                     kv, fl = b * (ctx_len + 1) * row * 2, 2.0 * heads * (row + rank) * T * (T + 1) / 2
@@ -569,7 +569,9 @@ def design_record(args):
                     kv, fl = b * (ctx_len + 1) * row * 2, 2.0 * heads * (row + rank) * T * (T + 1) / 2
                     a = cfg.layers[1]["mixer"]
                     by_entry = {"attn_bytes:pta_attn_talk_mfma": b * (ctx_len + 1) * a["kv_heads"] * (a["dim"] + a["vdim"]) * 2,
-                                "attn_flops:pta_attn_talk_mfma": 2.0 * (a["dim"] + a["vdim"]) * a["heads"] * T * (T + 1) / 2}
+                                "attn_flops:pta_attn_talk_mfma": 0.0}
+                    by_prompt = {"attn_bytes:pta_attn_talk_mfma": 0.0,
+                                 "attn_flops:pta_attn_talk_mfma": 2.0 * (a["dim"] + a["vdim"]) * a["heads"] * T * (T + 1) / 2}
                 elif name == "bimepel":  # keys and values of a token's own block of positions only
                     a = cfg.layers[0]["mixer"]
                     block = a["mask"]["size"]
@@ -599,6 +601,7 @@ def design_record(args):
                     model.step(cache, [slot], [prompt], "last")
                     cache.free(slot)
 
+                ops.timing_hint.update(by_prompt)
                 r[f"kernels_prefill_{T}"] = kernel_figures(model, ops, args.dtype, step, attn_flops=fl)
                 for key in by_entry:
                     ops.timing_hint.pop(key, None)

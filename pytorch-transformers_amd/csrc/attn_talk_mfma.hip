@@ -11,18 +11,34 @@ PTA_TALK_HEAD(1) PTA_TALK_HEAD(2) PTA_TALK_HEAD(3) PTA_TALK_HEAD(4) PTA_TALK_HEA
 PTA_TALK_HEAD(8)
 #undef PTA_TALK_HEAD
 
-// heads a wave holds: as many as the head size allows, all of one KV head, with at most sixteen waves; 0: none fits
-static int talk_heads_per_wave(int nh, int nkv, int d) {
+// heads a wave holds: as many as the head size allows, all of one KV head, with at most sixteen waves; 0: none fits.
+// heads_wg: the heads of a workgroup: all of them where the scores are mixed over the heads; without a mix the heads
+// of one KV head (or sixteen waves' worth of them), so that a token's heads spread over several workgroups.
+static int talk_heads_per_wave(int nh, int nkv, int d, bool mixed, int* heads_wg) {
     if (nh <= 0 || nkv <= 0 || nh % nkv || d % 16 || d < 16 || d > 128) return 0;
-    if ((size_t)nh * 4096 > 128 * 1024) return 0;  // the heads' tiles of two blocks of keys in LDS
+    if (mixed && (size_t)nh * 4096 > 128 * 1024) return 0;  // the heads' tiles of two blocks of keys in LDS
     const int g = nh / nkv;
     // PTA_TALK_HEADS: fewer heads a wave than the head size allows, for measurements (16 heads of 128 with a head a
     // wave on sixteen waves: 156 us a layer of 2,048 tokens against 107 with two heads a wave on eight; every wave reads
     // all heads' tiles, so twice the waves read twice as much from LDS)
     static const int most_env = getenv("PTA_TALK_HEADS") ? atoi(getenv("PTA_TALK_HEADS")) : 0;
     const int most = most_env > 0 ? std::min(most_env, talk_max_heads(d / 16)) : talk_max_heads(d / 16);
-    for (int ct = most; ct >= 1; ct /= 2)
-        if (g % ct == 0 && nh / ct <= 16) return ct;
+    for (int ct = most; ct >= 1; ct /= 2) {
+        if (g % ct) continue;
+        if (mixed) {
+            if (nh / ct > 16) continue;
+            if (heads_wg) *heads_wg = nh;
+            return ct;
+        }
+        int waves = g / ct;  // of one KV head; more than sixteen are cut into equal parts
+        while (waves > 16) {
+            int f = 2;
+            while (waves % f) ++f;
+            waves /= f;
+        }
+        if (heads_wg) *heads_wg = waves * ct;
+        return ct;
+    }
     return 0;
 }
 
@@ -34,7 +50,15 @@ extern "C" int pta_attn_talk_prompt_ranges(int tiles, int keys_seen) {
     return std::max(1, std::min({4, units / tiles, keys_seen / 128}));
 }
 
-extern "C" int pta_attn_talk_mfma_supported(int nh, int nkv, int d) { return talk_heads_per_wave(nh, nkv, d) > 0; }
+// mixed: whether the scores are mixed over the heads (then a workgroup holds all heads of its tokens)
+extern "C" int pta_attn_talk_mfma_supported(int nh, int nkv, int d, int mixed) {
+    return talk_heads_per_wave(nh, nkv, d, mixed != 0, nullptr) > 0;
+}
+// workgroups that share a token's heads in a launch
+extern "C" int pta_attn_talk_mfma_workgroups(int nh, int nkv, int d, int mixed) {
+    int heads_wg = 0;
+    return talk_heads_per_wave(nh, nkv, d, mixed != 0, &heads_wg) > 0 ? nh / heads_wg : 0;
+}
 
 extern "C" int pta_attn_talk_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                                   int bt_stride, const int* cu_tokens, const int* seq_start, const float* talk, float softcap,
@@ -43,7 +67,8 @@ extern "C" int pta_attn_talk_mfma(void* out, const void* q, const void* k_pool, 
                                   const float* head_bias, int weights_kind, void* stream) {
     PTA_REQUIRE(weights_kind == PTA_WEIGHTS_SOFTMAX || weights_kind == PTA_WEIGHTS_SIGMOID, "attn_talk_mfma: weights of kind %d are not built", weights_kind);
     PTA_REQUIRE(n_seqs > 0 && max_new > 0 && M > 0, "attn_talk_mfma: sizes must be positive");
-    const int ct = talk_heads_per_wave(nh, nkv, d);
+    int heads_wg = 0;
+    const int ct = talk_heads_per_wave(nh, nkv, d, talk != nullptr, &heads_wg);
     PTA_REQUIRE(ct > 0, "attn_talk_mfma: %d heads on %d KV heads of size %d are not built (sizes 16..128 in steps of 16, "
                 "at most 32 heads, at most 16 groups of heads that fit a wave)", nh, nkv, d);
     PTA_REQUIRE(window >= 0 && chunk >= 0 && softcap >= 0.f, "attn_talk_mfma: window, chunk and softcap are 0 (none) or positive");
@@ -59,7 +84,7 @@ extern "C" int pta_attn_talk_mfma(void* out, const void* q, const void* k_pool, 
     const float pre_mul = softcap > 0.f ? 2.0f * scale * TALK_LOG2E / softcap : scale;
     const TalkLaunch a{(bf16_t*)out, po, pm, pl, (const bf16_t*)q, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_table,
                        bt_stride, cu_tokens, seq_start, talk, softcap, pre_mul, n_seqs, max_new, nh, nkv, window, chunk,
-                       split_size, n_splits, (hipStream_t)stream, head_scale, head_bias, weights_kind};
+                       split_size, n_splits, (hipStream_t)stream, head_scale, head_bias, weights_kind, heads_wg};
     bool built = false;
     switch (d / 16) {
 #define PTA_TALK_CASE(DT_) case DT_: built = talk_launch_head<DT_>(a, ct); break;

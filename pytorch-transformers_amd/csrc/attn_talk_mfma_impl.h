@@ -6,7 +6,8 @@
 //    weight is sigmoid(s_h + head_bias[h]), not normalised over the keys, in place of the softmax)
 //
 // The mix needs every head's score of a (query, key) pair in one place.  A workgroup owns sixteen consecutive tokens
-// of one sequence and all heads; a wave owns CT heads of one KV head.  Keys are walked 32 at a time:
+// of one sequence and all heads (without a mix: the heads of one KV head, or a part of them, heads_wg of them, and
+// gridDim.z such workgroups share the tokens); a wave owns CT heads of one KV head.  Keys are walked 32 at a time:
 //
 //   S_h^T[32 keys x 16 tokens] = K[32 x d] . Q_h^T[d x 16]      per head of the wave, then scale and cap (32-bit)
 //   every wave leaves its heads' capped tiles in LDS, in the accumulator's own lane layout; after a barrier it
@@ -58,7 +59,7 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
     const int* __restrict__ block_table, int bt_stride, const int* __restrict__ cu_tokens,
     const int* __restrict__ seq_start, const float* __restrict__ talk, float cap, float pre_mul, int nh, int nkv,
     int window, int chunk, int split_size, int n_splits, const float* __restrict__ head_scale,
-    const float* __restrict__ head_bias, int weights_kind) {
+    const float* __restrict__ head_bias, int weights_kind, int heads_wg) {
     constexpr int D = DT * 16, DS = (DT + 1) / 2, CHUNKS = D / 8;
     extern __shared__ __attribute__((aligned(16))) float4 talk_tiles[];  // [2][nh][2][64], then the mix [nh][nh]
     auto lowest_key = [&](int t) {
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(64 * MAXW) void attn_talk_mfma_kernel(
     const int t0 = cu_tokens[seq], n_new = cu_tokens[seq + 1] - t0, start = seq_start[seq];
     const int tok0 = (int)(gridDim.x - 1 - blockIdx.x) * 16;  // late tokens, which see the most keys, start first
     if (tok0 >= n_new) return;
-    const int g = nh / nkv, h0 = wave * CT, kvh = h0 / g;
+    const int g = nh / nkv, h0 = blockIdx.z * heads_wg + wave * CT, kvh = h0 / g;
     const int tok = t0 + min(tok0 + c, n_new - 1);
     const int qpos = tok0 + c < n_new ? start + tok0 + c : -1;  // -1: a column that does not exist sees no key
     const int first_pos = start + tok0, last_pos = start + min(tok0 + 15, n_new - 1);
@@ -328,7 +329,7 @@ struct TalkLaunch {
     const int *cu_tokens, *seq_start; const float* talk; float cap, pre_mul;
     int n_seqs, max_new, nh, nkv, window, chunk, split_size, n_splits;
     hipStream_t s;
-    const float *head_scale, *head_bias; int weights_kind;
+    const float *head_scale, *head_bias; int weights_kind, heads_wg;
 };
 
 // heads that one wave may hold at this head size (the registers of the sums set it)
@@ -347,17 +348,17 @@ static void talk_launch_one(const TalkLaunch& a) {
             told[dev] = true;
         }
     }
-    const dim3 grid((a.max_new + 15) / 16, a.n_seqs * a.n_splits);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * (a.nh / CT)), lds, a.s, a.out, a.po, a.pm, a.pl, a.q, a.k_pool, a.v_pool,
+    const dim3 grid((a.max_new + 15) / 16, a.n_seqs * a.n_splits, a.nh / a.heads_wg);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * (a.heads_wg / CT)), lds, a.s, a.out, a.po, a.pm, a.pl, a.q, a.k_pool, a.v_pool,
                        a.block_table, a.bt_stride, a.cu_tokens, a.seq_start, a.talk, a.cap, a.pre_mul, a.nh, a.nkv, a.window,
-                       a.chunk, a.split_size, a.n_splits, a.head_scale, a.head_bias, a.weights_kind);
+                       a.chunk, a.split_size, a.n_splits, a.head_scale, a.head_bias, a.weights_kind, a.heads_wg);
 }
 
 // What pta_attn_talk_mfma launches for heads of DT x 16 elements with `ct` heads a wave; every head size is a
 // translation unit of its own (attn_talk_mfma_dt*.hip).  false: that combination is not built.
 template <int DT>
 bool talk_launch_head(const TalkLaunch& a, int ct) {
-    const int waves = a.nh / ct;
+    const int waves = a.heads_wg / ct;
 #define TALK_CASE(CT_)                                          \
     if (ct == CT_) {                                            \
         if (waves <= 8) talk_launch_one<DT, CT_, 8>(a);         \

@@ -108,6 +108,20 @@ __global__ void xielu_kernel(T* __restrict__ out, const T* __restrict__ z, long 
     Io<T>::st(out + i, xielu_value(Io<T>::ld(z + m * z_ld + f), softplus_f32(act[0]), 0.5f + softplus_f32(act[1])));
 }
 
+// bfloat16 rows of a multiple of eight elements at sixteen-byte addresses: eight elements a thread
+__global__ void xielu_bf16x8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ z, long z_ld, int F8, long n8,
+                                    const float* __restrict__ act) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n8) return;
+    const long m = i / F8, f = (i - m * F8) * 8;
+    const float ap = softplus_f32(act[0]), an = 0.5f + softplus_f32(act[1]);
+    float v[8];
+    unpack8(*reinterpret_cast<const uint4*>(z + m * z_ld + f), v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = xielu_value(v[e], ap, an);
+    *reinterpret_cast<uint4*>(out + m * (long)F8 * 8 + f) = pack8(v);
+}
+
 extern "C" int pta_xielu(void* out, const void* z, long z_ld, int M, int F, const float* act, int dtype, void* stream) {
     PTA_REQUIRE(M > 0 && F > 0 && out && z && act && z_ld >= F, "xielu: sizes must be positive and pointers given");
     PTA_REQUIRE(dtype == PTA_F32 || dtype == PTA_BF16, "xielu: unknown dtype %d", dtype);
@@ -116,6 +130,9 @@ extern "C" int pta_xielu(void* out, const void* z, long z_ld, int M, int F, cons
     const dim3 grid((unsigned)((n + 255) / 256));
     if (dtype == PTA_F32)
         hipLaunchKernelGGL(xielu_kernel<float>, grid, dim3(256), 0, s, (float*)out, (const float*)z, z_ld, F, n, act);
+    else if (F % 8 == 0 && z_ld % 8 == 0 && ((uintptr_t)z % 16) == 0 && ((uintptr_t)out % 16) == 0)
+        hipLaunchKernelGGL(xielu_bf16x8_kernel, dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0, s, (bf16_t*)out,
+                           (const bf16_t*)z, z_ld, F / 8, n / 8, act);
     else
         hipLaunchKernelGGL(xielu_kernel<bf16_t>, grid, dim3(256), 0, s, (bf16_t*)out, (const bf16_t*)z, z_ld, F, n, act);
     return pta_check_launch("xielu");

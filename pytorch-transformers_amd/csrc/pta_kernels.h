@@ -355,7 +355,8 @@ int pta_attn_talk(void* out, const void* q, const void* k_pool, const void* v_po
                   int dtype, void* stream);
 // The same on the matrix cores (bfloat16; attn_talk_mfma.hip): a step's tokens by sequence (cu_tokens, seq_start) as
 // pta_attn_mfma takes them; with one token per sequence the keys may be cut into n_splits ranges of split_size.
-int pta_attn_talk_mfma_supported(int nh, int nkv, int d);
+int pta_attn_talk_mfma_supported(int nh, int nkv, int d, int mixed);   // mixed: the scores are mixed over the heads
+int pta_attn_talk_mfma_workgroups(int nh, int nkv, int d, int mixed);  // workgroups that share a token's heads
 int pta_attn_talk_prompt_ranges(int tiles, int keys_seen);  // runs into which a prompt launch cuts every tile's keys
 int pta_attn_talk_mfma(void* out, const void* q, const void* k_pool, const void* v_pool, const int* block_table,
                        int bt_stride, const int* cu_tokens, const int* seq_start, const float* talk, float softcap,

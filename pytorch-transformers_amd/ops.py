@@ -703,10 +703,11 @@ def attention(q: torch.Tensor, k_pool, v_pool, block_table, ctx, slopes, scale: 
                         bias_of, bias_scale, chunk)
 
 
-def attn_talk_mfma_ok(q: torch.Tensor, nkv: int) -> bool:
-    """Whether the matrix-core kernel for capped, mixed scores takes these queries (bfloat16, sizes built)."""
+def attn_talk_mfma_ok(q: torch.Tensor, nkv: int, mixed: bool = True) -> bool:
+    """Whether the matrix-core kernel for capped, mixed scores takes these queries (bfloat16, sizes built); ``mixed``:
+    whether the scores are mixed over the heads (without a mix a token's heads need not share a workgroup)."""
     return q.dtype == torch.bfloat16 and bool(
-        load_library().pta_attn_talk_mfma_supported(int(q.shape[1]), int(nkv), int(q.shape[2])))
+        load_library().pta_attn_talk_mfma_supported(int(q.shape[1]), int(nkv), int(q.shape[2]), int(bool(mixed))))
 
 
 def attn_talk_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_start, scale: float, *, max_new: int,
@@ -740,14 +741,15 @@ def attn_talk_mfma(q: torch.Tensor, k_pool, v_pool, block_table, cu_tokens, seq_
     return out
 
 
-def talk_decode_ranges(n_seqs: int, max_len: int, window: int = 0, chunk: int = 0) -> tuple:
+def talk_decode_ranges(n_seqs: int, max_len: int, window: int = 0, chunk: int = 0, per_token: int = 1) -> tuple:
     """(runs, 0) for a decode step of ``attn_talk_mfma``: every token cuts the keys it sees into so many equal runs of
     blocks, about two workgroups for every compute unit, a run no shorter than a page at the longest context, at most
     1,024 runs and 65,535 workgroups a launch.  The size 0 says that the runs are each token's own (``attn_talk_mfma``):
     what a window has left behind is in no run, so the partial results do not grow with the context.  The batch counts
     by its next power of two and the longest context by its next multiple of 1,024, so that a captured step, which is
-    sized for a padded batch and such a bound, is cut exactly as the same step run directly."""
-    n_seqs = 1 << max(int(n_seqs) - 1, 0).bit_length()
+    sized for a padded batch and such a bound, is cut exactly as the same step run directly.  ``per_token``: the
+    workgroups that share a token's heads (more than one where the scores are not mixed over the heads)."""
+    n_seqs = (1 << max(int(n_seqs) - 1, 0).bit_length()) * max(1, int(per_token))
     max_len = (int(max_len) + 1023) // 1024 * 1024
     seen = max_len
     for bound in (window, chunk):
@@ -763,13 +765,16 @@ def attention_talk(q: torch.Tensor, k_pool, v_pool, block_table, ctx, scale: flo
     softmax: picks the kernel for the step's shape and type.  bfloat16 with sizes the matrix-core kernel is built
     for: that kernel, with the context cut into ranges when every sequence brings one token; anything else: the
     32-bit kernel."""
-    if attn_talk_mfma_ok(q, k_pool.shape[1]):
+    if attn_talk_mfma_ok(q, k_pool.shape[1], talk is not None):
         n_splits, size = 1, ATTN_SPLIT_KEYS
+        per_token = int(load_library().pta_attn_talk_mfma_workgroups(int(q.shape[1]), int(k_pool.shape[1]), int(q.shape[2]),
+                                                                     int(talk is not None)))
         if ctx.is_decode:
-            n_splits, size = talk_decode_ranges(ctx.n_seqs, ctx.max_len, window, chunk)
+            n_splits, size = talk_decode_ranges(ctx.n_seqs, ctx.max_len, window, chunk, per_token)
+            n_splits = min(n_splits, 65535 // max(1, ctx.n_seqs))
         else:  # few tiles of sixteen tokens: each cuts its keys into runs, so that no compute unit idles
             seen = min([ctx.max_len] + [b + 15 for b in (window, chunk) if b > 0])
-            tiles = sum((n + 15) // 16 for n in ctx.new_tokens)
+            tiles = sum((n + 15) // 16 for n in ctx.new_tokens) * per_token
             n_splits, size = int(load_library().pta_attn_talk_prompt_ranges(tiles, seen)), 0
         return attn_talk_mfma(q, k_pool, v_pool, block_table, ctx.cu_tokens, ctx.seq_start, scale,
                               max_new=max(ctx.new_tokens), talk=talk, softcap=softcap, window=window, chunk=chunk,

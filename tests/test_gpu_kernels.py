@@ -1243,9 +1243,13 @@ def test_attn_talk_mfma_decode_ranges(nh, nkv, d, ranges):
 def test_attn_talk_mfma_sizes():
     ops = _ops()
     lib = ops.load_library()
-    assert lib.pta_attn_talk_mfma_supported(16, 8, 128) and lib.pta_attn_talk_mfma_supported(32, 8, 128)
-    assert not lib.pta_attn_talk_mfma_supported(8, 4, 40) and not lib.pta_attn_talk_mfma_supported(8, 4, 256)
-    assert not lib.pta_attn_talk_mfma_supported(34, 34, 64) and not lib.pta_attn_talk_mfma_supported(64, 8, 64)
+    assert lib.pta_attn_talk_mfma_supported(16, 8, 128, 1) and lib.pta_attn_talk_mfma_supported(32, 8, 128, 1)
+    assert not lib.pta_attn_talk_mfma_supported(8, 4, 40, 1) and not lib.pta_attn_talk_mfma_supported(8, 4, 256, 1)
+    assert not lib.pta_attn_talk_mfma_supported(34, 34, 64, 1) and not lib.pta_attn_talk_mfma_supported(64, 8, 64, 1)
+    # scores that are not mixed over the heads: a token's heads spread over workgroups, so their number is no bound
+    assert lib.pta_attn_talk_mfma_supported(64, 8, 64, 0) and lib.pta_attn_talk_mfma_workgroups(64, 8, 64, 0) == 8
+    assert lib.pta_attn_talk_mfma_workgroups(16, 8, 128, 1) == 1 and lib.pta_attn_talk_mfma_workgroups(34, 34, 64, 0) == 34
+    assert lib.pta_attn_talk_mfma_workgroups(68, 1, 16, 0) == 17  # seventeen waves of four heads: a wave a workgroup
     assert lib.pta_attn_talk_prompt_ranges(128, 2048) in (1, 2) and lib.pta_attn_talk_prompt_ranges(4096, 2048) == 1
     assert lib.pta_attn_talk_prompt_ranges(4, 100) == 1 and lib.pta_attn_talk_prompt_ranges(8, 5000) == 4
     for n, length, window in ((1, 1, 0), (8, 1025, 1024), (64, 5000, 0), (3, 300000, 0), (512, 100, 70), (1, 70000, 1024),
