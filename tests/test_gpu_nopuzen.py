@@ -583,3 +583,49 @@ def test_configurations_drawn_at_random(tmp_path, seed):
             got = helpers.run_schedule(rp, records)
             for rid in reqs:
                 assert_model_close(got[rid], want[rid], rel, f"{json.dumps(cfg)} {dtype} {label} {rid}")
+
+
+def draw_larger_config(seed):
+    """Sizes that the matrix-core kernels and the products for batches of rows take: heads of 32 to 128 elements, latents of
+    64 to 256, experts of 64 and 128 rows on widths that are multiples of 64."""
+    import random
+
+    r = random.Random(1000 + seed)
+    layers = []
+    for i in range(r.randint(2, 3)):
+        if (i + seed) % 2 == 0:
+            dr = r.choice([16, 32, 64])
+            a = latent(r.choice([4, 6, 12]), r.choice([32, 64, 96, 128]), dr, r.choice([32, 64, 128]), r.choice([64, 96, 256]),
+                       r.choice([64, 160]), r.choice([0.08, 0.12]), r.choice([10000.0, 500000.0]), r.random() < 0.7)
+        else:
+            kv, d = r.choice([1, 2, 4]), r.choice([32, 48, 64, 128])
+            a = attn(kv * r.choice([1, 2, 4]), kv, d, r.choice([32, 64, 80]), r.choice([0.1, 0.15]), r.choice([0.0, 12.0, 30.0]),
+                     r.choice([d // 2, d]), r.choice([10000.0, 1000000.0]), r.random() < 0.3)
+        kind = r.choice(["dense", "moe"])
+        if kind == "dense":
+            a = dense(a, r.choice([192, 448]))
+        else:
+            count, size = r.choice([2, 4]), r.choice([2, 6])
+            keep = r.randint(1, count)
+            a = moe(a, r.choice([64, 128]), count * size, r.randint(1, min(6, keep * size)), r.choice([1.0, 2.5]), (count, keep),
+                    r.choice([0, 64, 192]))
+        layers.append(a)
+    return config(layers, vocab=r.choice([300, 513]), width=r.choice([128, 192, 320]), eps=r.choice([1e-5, 1e-6]))
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_larger_configurations_drawn_at_random(tmp_path, seed):
+    from pytorch_transformers_amd.engine.replay import Replayer
+
+    cfg = draw_larger_config(seed)
+    w = make_weights(cfg, seed=seed)
+    reqs = helpers.make_requests(cfg["vocab"], [150, 9, 40, 70], seed=seed)
+    want = plain_all(cfg, w, reqs)
+    folder = write_model(tmp_path / "m", cfg, w)
+    for dtype, rel in (("float32", helpers.REL_F32), ("bfloat16", REL_BF16_MODEL)):
+        rp = Replayer(load(folder, dtype), 1024, max_slots=4)
+        for label, records in (("whole", helpers.schedule_whole(reqs)), ("tail", helpers.schedule_tail(reqs, 20)),
+                               ("batches", helpers.schedule_batches(reqs, 4, decode=(4, 1, 7)))):
+            got = helpers.run_schedule(rp, records)
+            for rid in reqs:
+                assert_model_close(got[rid], want[rid], rel, f"{json.dumps(cfg)} {dtype} {label} {rid}")
