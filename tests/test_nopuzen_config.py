@@ -115,3 +115,25 @@ def test_layers_that_keep_the_same_rows_share_a_page_pool():
     c, d = groups[runs[1][1]], groups[runs[4][1]]
     assert runs[1][1] == runs[5][1] and c.values and c.kv_heads == 2 and c.head_dim == 32 and c.num_layers == 2
     assert d.values and d.head_dim == 48 and d.num_layers == 1
+
+
+@pytest.mark.parametrize("dims,base,scaling", [(8, 10000.0, None), (16, 50.0, {"factor": 4.0, "original": 64, "fast": 8.0, "slow": 1.0}),
+                                               (64, 500000.0, {"factor": 16.0, "original": 4096, "fast": 32.0, "slow": 1.0}),
+                                               (2, 100.0, {"factor": 2.0, "original": 8, "fast": 1.0, "slow": 1.0}),
+                                               (12, 10000.0, {"factor": 8.0, "original": 100000, "fast": 64.0, "slow": 0.5})])
+def test_the_builders_frequencies_are_the_plain_ones(dims, base, scaling):
+    """The table a mixer rotates by, and what its cosines and sines are multiplied by, against the plain formulas: no
+    ramp, a ramp inside the table, a ramp that is clamped at either end."""
+    import plain_nopuzen as P
+    from pytorch_transformers_amd.engine.nopuzen import _positions
+
+    rot = {"base": base, "dims": dims}
+    if scaling:
+        rot["scaling"] = scaling
+    for pairing in ("half", "interleaved"):
+        r = _positions(rot, dims + 4, pairing).rotation()
+        want = P.rotary_frequencies(rot)
+        assert r.rotary_dim == dims and r.pairing == pairing
+        assert float((r.inv_freq.double() - want).abs().max()) <= 1e-7 * float(want.abs().max())
+        assert abs(r.scale - P.rotary_magnitude(rot)) < 1e-12
+    assert _positions(None, 16, "half").rotation() is None
