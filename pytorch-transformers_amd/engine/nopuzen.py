@@ -80,7 +80,8 @@ def build_nopuzen(cfg: NopuzenConfig) -> ModelSpec:
         ffn = norm2 = None
         if layer.get("mlp") is not None:
             ffn, norm2 = _feed_forward(cfg, f"{p}.mlp", layer["mlp"]), _norm(f"{p}.norm2", cfg)
-        blocks.append(PostNormBlock(mixer, ffn, _norm(f"{p}.norm1", cfg), norm2))
+        # (the last layer's last norm and addition ride in the final norm's launch)
+        blocks.append(PostNormBlock(mixer, ffn, _norm(f"{p}.norm1", cfg), norm2, hand_on_unformed=i == len(cfg.layers) - 1))
         if isinstance(mixer, LatentAttentionMixer):
             key = ("latent", 1, mixer.cache_row)
         else:

@@ -133,18 +133,22 @@ class PostNormBlock(Part):
     whatever the compute type (``WideResidual``): a sublayer reads its copy in the compute type, the norm, the
     scaling and the addition are one 32-bit launch that also writes that copy for the next sublayer.
     ``feed_forward`` may be None (a layer of the mixer alone).  With ``depth_mix`` (``parts.depth.DepthMix``) the
-    block's result is kept as the next of the step's streams and what goes on is their weighted sum."""
+    block's result is kept as the next of the step's streams and what goes on is their weighted sum.  ``hand_on_unformed``
+    (for a model's last block, with LayerNorms): the last sublayer's output goes on not yet normed and added
+    (``PendingNormSum``), and the final norm's launch does both on its way, for the rows whose logits are wanted alone."""
 
     accepts_sum = False
     accepts_wide = True
 
     def __init__(self, mixer: Part, feed_forward: Optional[Part], norm_mixer: Part, norm_ffn: Optional[Part],
-                 residual_mult: float = 1.0, depth_mix: Optional[Part] = None):
+                 residual_mult: float = 1.0, depth_mix: Optional[Part] = None, hand_on_unformed: bool = False):
         if (feed_forward is None) != (norm_ffn is None):
             raise ValueError("a feed-forward and its norm come together or not at all")
         self.mixer, self.feed_forward, self.norm_mixer, self.norm_ffn = mixer, feed_forward, norm_mixer, norm_ffn
         self.residual_mult = float(residual_mult)
         self.depth_mix = depth_mix
+        last_norm = norm_mixer if norm_ffn is None else norm_ffn
+        self.hand_on_unformed = bool(hand_on_unformed) and depth_mix is None and hasattr(last_norm, "affine")
 
     def children(self) -> Sequence[Part]:
         return tuple(p for p in (self.norm_mixer, self.norm_ffn, self.mixer, self.feed_forward, self.depth_mix)
@@ -178,10 +182,14 @@ class PostNormBlock(Part):
         # the launch that forms the block's result also keeps it as a stream and goes on to the streams' weighted sum
         mix = self.depth_mix.fused(history) if keep is not None else None
         mixed = self.mixer.forward(x.narrow, ctx, call)
+        if last and self.hand_on_unformed:
+            return PendingNormSum(x.wide, mixed, self.norm_mixer.affine(), self.residual_mult, self.norm_mixer.eps, ctx.dtype)
         narrow, wide = self.norm_mixer.apply(mixed, ctx.dtype, residual=x.wide, mult=self.residual_mult, want_wide=True,
                                              out_wide=keep if last else None, mix=mix if last else None)
         if not last:
             out = self.feed_forward.forward(narrow, ctx)
+            if self.hand_on_unformed:
+                return PendingNormSum(wide, out, self.norm_ffn.affine(), self.residual_mult, self.norm_ffn.eps, ctx.dtype)
             narrow, wide = self.norm_ffn.apply(out, ctx.dtype, residual=wide, mult=self.residual_mult, want_wide=True,
                                                out_wide=keep, mix=mix)
         return WideResidual(wide, narrow, history)
