@@ -104,14 +104,13 @@ class LatentAttentionMixer(Part):
                                  "half" if rot is None else rot.pairing, ctx.token_pos, ctx.token_seq, table, k_pool,
                                  self.heads, self.dim, self.rot_dim, self.rank, write_cache=call.write_cache, q=queries)
         gate = proj[:, at + D:at + D + H * self.value_dim] if self.gate else None
-        proj = queries
         library = x.dtype == torch.bfloat16 and M > ops.HEAD_PROJECT_LIBRARY_ROWS
         # each head's plain query through the transpose of its key expansion: the first `rank` of its frame
         if library:
-            plain = proj[:, :H * (self.dim + self.rot_dim)].unflatten(1, (H, self.dim + self.rot_dim))[:, :, :self.dim]
+            plain = queries.unflatten(1, (H, self.dim + self.rot_dim))[:, :, :self.dim]
             q_full[:, :, :self.rank].copy_(ops.head_project_library(plain, self.k_side, torch.float32).transpose(0, 1))
         else:
-            ops.head_project(proj, self.dim + self.rot_dim, self.k_side, H, self.dim, self.rank,
+            ops.head_project(queries, self.dim + self.rot_dim, self.k_side, H, self.dim, self.rank,
                              out=q_full.view(M, H * D), out_head=D)
         lat = ops.attn_latent(q_full, k_pool, table, ctx.token_seq, ctx.token_pos, self.rank, self.scale, ctx=ctx)
         if library:
